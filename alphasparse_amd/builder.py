@@ -45,6 +45,13 @@ def _bind(L):
     L.as_builder_algorithmic_bytes.restype = C.c_int64
     L.as_builder_algorithmic_bytes.argtypes = [vp]
     L.as_hip_device_count.restype = C.c_int
+    L.as_builder_spmv_device.argtypes = [vp, vp, vp]
+    L.as_builder_clears_y.argtypes = [vp]
+    L.as_hip_last_error.restype = C.c_char_p
+    L.as_hip_alloc.argtypes = [C.POINTER(vp), C.c_uint64]
+    L.as_hip_free.argtypes = [vp]
+    L.as_hip_h2d.argtypes = [vp, vp, C.c_uint64]
+    L.as_hip_d2h.argtypes = [vp, vp, C.c_uint64]
     _bound = True
 
 
@@ -187,6 +194,33 @@ class Builder:
         y = np.zeros(self.rows, dtype=x.dtype)
         self._chk(self._L.as_builder_spmv(self._h, x.ctypes.data_as(C.c_void_p), y.ctypes.data_as(C.c_void_p)))
         return y
+
+    def spmv_device(self, x, y_before=None):
+        """y = A x on device buffers of the caller (as_builder_spmv_device): y
+        holds `y_before` (a scalar or an array; default NaN) when the call starts, so a row that no kernel writes,
+        or a sum added to what was there, shows."""
+        L = self._L
+        x = np.ascontiguousarray(x)
+        if len(x) != self.cols:
+            raise ValueError("x has %d entries, matrix has %d columns" % (len(x), self.cols))
+        y = np.full(self.rows, np.nan if y_before is None else y_before, dtype=x.dtype)
+        dx, dy = C.c_void_p(), C.c_void_p()
+        if L.as_hip_alloc(C.byref(dx), x.nbytes) != 0 or L.as_hip_alloc(C.byref(dy), y.nbytes) != 0:
+            raise capi.AlphaSparseError(L.as_hip_last_error().decode())
+        try:
+            if L.as_hip_h2d(dx, x.ctypes.data_as(C.c_void_p), x.nbytes) != 0 or L.as_hip_h2d(dy, y.ctypes.data_as(C.c_void_p), y.nbytes) != 0:
+                raise capi.AlphaSparseError(L.as_hip_last_error().decode())
+            self._chk(L.as_builder_spmv_device(self._h, dx, dy))
+            if L.as_hip_d2h(y.ctypes.data_as(C.c_void_p), dy, y.nbytes) != 0:
+                raise capi.AlphaSparseError(L.as_hip_last_error().decode())
+        finally:
+            L.as_hip_free(dx)
+            L.as_hip_free(dy)
+        return y
+
+    def clears_y(self):
+        """True when an SpMV of the current templates starts with a clear of y."""
+        return bool(self._chk(self._L.as_builder_clears_y(self._h)))
 
     def set_x(self, x):
         x = np.ascontiguousarray(x)

@@ -197,6 +197,13 @@ int as_builder_spmv_device(as_builder *b, const void *x_dev, void *y_dev) {
   AS_API_END(-1)
 }
 
+int as_builder_clears_y(as_builder *b) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b, "null builder");
+  return asx::y_needs_clear(*b->b) ? 1 : 0;
+  AS_API_END(-1)
+}
+
 int as_builder_set_x(as_builder *b, const void *x_host) {
   AS_API_BEGIN
   AS_CHECK(b && b->b && x_host && b->b->device_ready, "builder is not on the device");
@@ -393,7 +400,7 @@ static asx::CooInput coo_of(const as_matrix *m) {
 int as_part_execute_code_builder(as_builder *b, const int64_t *sub_matrix_ids, uint64_t n_ids, uint64_t repeat,
                                  float *time_ms, float *gflops) {
   AS_API_BEGIN
-  AS_CHECK(b && b->b && time_ms && gflops && repeat > 0, "bad argument");
+  AS_CHECK(b && b->b && time_ms && gflops, "bad argument");
   asx::Builder &bd = *b->b;
   AS_CHECK(bd.device_ready, "builder is not on the device");
   // run only the listed sub-matrices: the templates of the others are parked for the call
@@ -415,6 +422,14 @@ int as_part_execute_code_builder(as_builder *b, const int64_t *sub_matrix_ids, u
     }
   } restore{bd, parked, changed};
   if (changed) asx::invalidate_module(bd);
+  if (repeat == 0) {
+    // the reference's own count (executor.cc:247-255): 185.2 G padded elements in all, at least two launches
+    uint64_t total_nnz = 0;
+    for (auto &k : bd.subs)
+      if (k.tpl) total_nnz += k.tpl->padding_arr_size;
+    AS_CHECK(total_nnz > 0, "no sub-matrix has a template");
+    repeat = std::max<uint64_t>(2, 185200000000ull / total_nnz);
+  }
   asx::time_spmv(bd, repeat, true, *time_ms, *gflops);  // kernel; synchronize -- as the upstream timing loop
   return 0;
   AS_API_END(-1)

@@ -27,6 +27,7 @@ struct SubKernel {
 struct Builder {
   const Matrix *matrix = nullptr;  // not owned; must outlive template initialisation
   uint64_t rows = 0, cols = 0, origin_nnz = 0;
+  bool rows_compacted = false;     // remove_empty_rows ran: y has rows that no kernel stores
   DType val_dtype = FLOAT;
   std::vector<SubKernel> subs;     // index = sub-matrix id; tpl == nullptr until set
   std::string source;
@@ -64,11 +65,16 @@ void compile_builder(Builder &b);                 // hipRTC, no GPU needed (comp
 // code objects kept by module source, and how often a compilation was answered from them
 void code_cache_stats(uint64_t &entries, uint64_t &hits);
 void load_and_upload(Builder &b, int device);     // module load + arrays to HBM (code_of_write_template_data_to_gpu)
-// y = A x on device buffers already holding x; y is cleared first.
+// True when y has to be cleared before the kernels run: a kernel adds into y (atomics), a row of y belongs to
+// no kernel (rows removed by remove_empty_rows, a sub-matrix without template) or holds no element.  Graphs whose
+// kernels store every row exactly once (ELL / SELL strips, the two-kernel LDS templates) skip the clear.
+bool y_needs_clear(const Builder &b);
+// y = A x on device buffers already holding x; y is cleared first where y_needs_clear says so.
 void launch_spmv(Builder &b, const void *x_dev, void *y_dev);
 void spmv_host(Builder &b, const void *x_host, void *y_host);
 // Timing: `reps` launches of all kernels.  sync_each_launch reproduces the
 // upstream loop (kernel; cudaDeviceSynchronize, code_builder.cc:1524-1557).
+// Every repetition is what launch_spmv issues (the clear of y included where needed).
 // Returns ms for all reps; gflops = 2 * origin_nnz * reps / time.
 void time_spmv(Builder &b, uint64_t reps, bool sync_each_launch, float &time_ms, float &gflops);
 // Bytes one SpMV moves with the chosen format (padded col/val + passed

@@ -59,6 +59,9 @@ struct Template {
   IArr col_index_arr;
   ValVec val_arr;
   uint64_t origin_nnz = 0;        // non-padding elements this kernel covers
+  // elements of the compressed sub-matrix with the padding of its operators (compressed_block_t::padding_arr_size,
+  // op_manager.cc:3789, 3933): what the executor sizes its default repeat count by (executor.cc:237)
+  uint64_t padding_arr_size = 0;
   // launch parameters (template_node params, exe_graph.hpp:411-475)
   uint64_t tblock_num = 0, thread_num_in_block = 0, thread_num_of_row_reduce = 1;
   // Rows (or TLBs) handled per lane with one wide load; 1, 2 or 4.  An MI355X
@@ -82,6 +85,9 @@ struct Template {
   // > 0: a second kernel `spmv_<sub>_finish` with this many workgroups follows spmv_<sub> on the same
   // stream (same arguments)
   uint64_t finish_tblock_num = 0, finish_thread_num = 256, finish_lds_bytes = 0;
+  // false: the kernels store every row of their strip of y exactly once and add to none, so y need not be
+  // cleared for them (set by add_template_to_builder through template_needs_cleared_y)
+  bool y_needs_clear = true;
 
   TArr *find(const std::string &n) {
     for (auto &t : arrays)
@@ -117,6 +123,9 @@ uint64_t effective_unit_num(const Matrix &m, uint64_t sub, const std::vector<uin
 // for the first `effective` units; returns whether a permutation was applied.
 bool apply_global_sort(const Matrix &m, uint64_t sub, std::vector<uint64_t> &unit_row, uint64_t effective);
 void init_template_common(Template &t, TemplateType type, const Matrix &m, uint64_t sub);
+// True when the kernels of `t` add into y anywhere (atomics on shared rows, on rows that cross a tile) or when a
+// row of the strip holds no element and is therefore stored by nobody: y must then be cleared before the launch.
+bool template_needs_cleared_y(const Template &t, const Matrix &m, uint64_t sub);
 
 // ---- per-family entry points ------------------------------------------------
 // is_supported_by_<T>, init_<T>, try_all_compress, code_of_template_kernal,

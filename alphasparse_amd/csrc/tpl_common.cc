@@ -80,6 +80,30 @@ void init_template_common(Template &t, TemplateType type, const Matrix &m, uint6
   t.kernal_first_row_index = m.items[sub].min_row;
   t.kernal_first_col_index = m.items[sub].min_col;
   t.origin_nnz = m.items[sub].end_coo - m.items[sub].begin_coo + 1;
+  const CompressedBlock &cb = *m.items[sub].cb;
+  t.padding_arr_size = cb.padding_val ? cb.padding_val->size() : (cb.val ? cb.val->size() : 0);
+}
+
+bool template_needs_cleared_y(const Template &t, const Matrix &m, uint64_t sub) {
+  if (t.is_atom_add) return true;
+  // the CSR5-like pair adds the partial sums of rows that cross a tile or a wavefront into y
+  if (t.type == UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE ||
+      t.type == UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE_WITH_WARP_REDUCE)
+    return true;
+  // the two-kernel LDS templates store every row of the strip in their finish kernel, with or without elements
+  if (t.finish_tblock_num && (t.type == SHARED_MEMORY_TILE_TEMPLATE || t.type == SHARED_MEMORY_PRODUCT_BIN_TEMPLATE))
+    return false;
+  // the row-wise templates store the rows that have a unit (TLB, WLB or BLB): a row without elements has none
+  const DenseItem &it = m.items[sub];
+  const uint64_t sub_rows = it.max_row - it.min_row + 1;
+  std::vector<bool> seen(sub_rows, false);
+  uint64_t count = 0;
+  for (uint64_t r : it.cb->read_index[0]->index_arr.v)
+    if (r < sub_rows && !seen[r]) {
+      seen[r] = true;
+      count++;
+    }
+  return count != sub_rows;
 }
 
 #define AS_DISPATCH(type, call)                                                                         \

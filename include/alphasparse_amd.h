@@ -245,10 +245,16 @@ const char *as_builder_kernel_source(as_builder *b);
 int as_builder_compile(as_builder *b);
 /* code_builder.cc:1248 code_of_write_template_data_to_gpu: module load + arrays into HBM */
 int as_builder_upload(as_builder *b, int device);
-/* y = A x, host vectors in the matrix value type; y is cleared first */
+/* y = A x, host vectors in the matrix value type.  y is cleared first by a fill kernel where the graph needs it
+ * (as_builder_clears_y): a kernel adds into y with atomics, or some row of y is stored by no kernel.  Graphs whose
+ * kernels store every row exactly once (ELL / SELL strips, the two-kernel LDS templates) launch no clear; whatever
+ * y held before the call is overwritten either way.  The reference's generated program clears y with
+ * cudaMemset before its timing loop only (code_builder.cc:1524-1557). */
 int as_builder_spmv(as_builder *b, const void *x_host, void *y_host);
 /* same on device pointers the caller owns */
 int as_builder_spmv_device(as_builder *b, const void *x_dev, void *y_dev);
+/* 1 when an SpMV of the builder's current templates starts with a clear of y, 0 when it does not; <0 error */
+int as_builder_clears_y(as_builder *b);
 /* 0 (default): the kernels of the sub-matrices run concurrently, one stream each (code_builder.cc:1517-1518);
  * 1: one after the other on the caller's stream.  No counterpart in the reference. */
 int as_builder_set_serial_launch(as_builder *b, int serial);
@@ -273,7 +279,9 @@ int as_builder_time(as_builder *b, uint64_t reps, int sync_each_launch, float *t
 /* bytes one SpMV moves with the chosen format: padded col+val, passed metadata, x once, y once (twice with atomics) */
 int64_t as_builder_algorithmic_bytes(as_builder *b);
 /* executor.hpp:12 part_execute_code_builder: run only the listed sub-matrices (n_ids = 0: all), `repeat` launches,
- * synchronising after each; returns 0 and (time_ms, gflops), <0 on failure (upstream: bool false) */
+ * synchronising after each; repeat = 0 takes the reference's own count, 185.2e9 / (padded elements of the listed
+ * sub-matrices), at least 2 (executor.cc:247-255).  Returns 0 and (time_ms for all launches, gflops), <0 on
+ * failure (upstream: bool false) */
 int as_part_execute_code_builder(as_builder *b, const int64_t *sub_matrix_ids, uint64_t n_ids, uint64_t repeat,
                                  float *time_ms, float *gflops);
 /* executor.hpp:19 execute_code_builder: final run sized to about `seconds` (executor.cc:191-208) */

@@ -60,6 +60,9 @@ def run_case(gpu, gen, vdt, dense, skel, kw, launches=({},), templates_filter=No
             print("case:", what, flush=True)
             assert_y(b.spmv(x), y_ref, mag, npd, what)
             assert_y(b.spmv(x), y_ref, mag, npd, what + " (second run: y must be re-zeroed)")
+            # a y full of NaN before the call: the clear is launched exactly where the graph needs it, and a
+            # graph without clear stores every row
+            assert_y(b.spmv_device(x), y_ref, mag, npd, what + " (y = NaN before the call, clear: %s)" % b.clears_y())
             b.close()
             ran += 1
     assert ran > 0
@@ -228,6 +231,8 @@ def test_spmv_with_empty_rows_removed(gpu, dense, skel, kw, vdt):
         assert len(y) == rows
         assert_y(y, y_ref, mag, npd, "%s %s" % (skel, K.TEMPLATE_NAMES[tp]))
         assert_y(b.spmv(x), y_ref, mag, npd, "%s second run" % skel)
+        assert b.clears_y()  # the rows that were removed are stored by no kernel
+        assert_y(b.spmv_device(x), y_ref, mag, npd, "%s y = NaN before the call" % skel)
         b.close()
 
 
@@ -423,6 +428,8 @@ def test_full_laplacian_matches_oracle(laplacian_full):
     assert rows == 4194304 and len(r) == 20963328
     y_ref, mag = oracle_y(rows, r, c, v, x)
     assert_y(b.spmv(x), y_ref, mag, np.float32, "C2 ELL")
+    assert not b.clears_y()  # direct stores, every row has elements: the SpMV is one kernel
+    assert_y(b.spmv_device(x), y_ref, mag, np.float32, "C2 ELL (y = NaN before the call)")
 
 
 def test_full_laplacian_closed_form_and_linearity(laplacian_full):
@@ -487,6 +494,9 @@ def test_full_size_tile_and_product_bin_graphs(gpu, make, capsys):
     y_ref, mag = oracle_y(rows, r, c, v, x)
     y1 = b.spmv(x)
     assert_y(y1, y_ref, mag, npd, make.__name__)
+    # C3 and C5 (a sorted tile strip + a product-bin strip) store every row once: no clear; C4 adds into y
+    assert b.clears_y() == (not long_strip)
+    assert_y(b.spmv_device(x), y_ref, mag, npd, make.__name__ + " (y = NaN before the call)")
     eps = np.finfo(npd).eps
     off = np.concatenate([[0], np.cumsum(np.bincount(np.asarray(r, np.int64), minlength=rows))])
     row_sum = np.add.reduceat(v.astype(np.float64), off[:-1])
