@@ -46,7 +46,10 @@ def _bind(L):
     L.as_builder_algorithmic_bytes.argtypes = [vp]
     L.as_hip_device_count.restype = C.c_int
     L.as_builder_spmv_device.argtypes = [vp, vp, vp]
+    L.as_builder_spmv_device_no_alloc.argtypes = [vp, vp, vp]
     L.as_builder_clears_y.argtypes = [vp]
+    L.as_builder_static_scratch_need.restype = C.c_int64
+    L.as_builder_static_scratch_need.argtypes = [vp]
     L.as_hip_last_error.restype = C.c_char_p
     L.as_hip_alloc.argtypes = [C.POINTER(vp), C.c_uint64]
     L.as_hip_free.argtypes = [vp]
@@ -195,8 +198,8 @@ class Builder:
         self._chk(self._L.as_builder_spmv(self._h, x.ctypes.data_as(C.c_void_p), y.ctypes.data_as(C.c_void_p)))
         return y
 
-    def spmv_device(self, x, y_before=None):
-        """y = A x on device buffers of the caller (as_builder_spmv_device): y
+    def spmv_device(self, x, y_before=None, no_alloc=False):
+        """y = A x on device buffers of the caller (as_builder_spmv_device, or as_builder_spmv_device_no_alloc): y
         holds `y_before` (a scalar or an array; default NaN) when the call starts, so a row that no kernel writes,
         or a sum added to what was there, shows."""
         L = self._L
@@ -210,7 +213,8 @@ class Builder:
         try:
             if L.as_hip_h2d(dx, x.ctypes.data_as(C.c_void_p), x.nbytes) != 0 or L.as_hip_h2d(dy, y.ctypes.data_as(C.c_void_p), y.nbytes) != 0:
                 raise capi.AlphaSparseError(L.as_hip_last_error().decode())
-            self._chk(L.as_builder_spmv_device(self._h, dx, dy))
+            call = L.as_builder_spmv_device_no_alloc if no_alloc else L.as_builder_spmv_device
+            self._chk(call(self._h, dx, dy))
             if L.as_hip_d2h(y.ctypes.data_as(C.c_void_p), dy, y.nbytes) != 0:
                 raise capi.AlphaSparseError(L.as_hip_last_error().decode())
         finally:
@@ -221,6 +225,10 @@ class Builder:
     def clears_y(self):
         """True when an SpMV of the current templates starts with a clear of y."""
         return bool(self._chk(self._L.as_builder_clears_y(self._h)))
+
+    def static_scratch_need(self):
+        """Bytes of the library's static scratch array the kernels would use in spmv_device(no_alloc=True)."""
+        return int(self._chk(self._L.as_builder_static_scratch_need(self._h)))
 
     def set_x(self, x):
         x = np.ascontiguousarray(x)

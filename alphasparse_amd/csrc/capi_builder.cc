@@ -197,6 +197,22 @@ int as_builder_spmv_device(as_builder *b, const void *x_dev, void *y_dev) {
   AS_API_END(-1)
 }
 
+int as_builder_spmv_device_no_alloc(as_builder *b, const void *x_dev, void *y_dev) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b && x_dev && y_dev, "null argument");
+  asx::launch_spmv_no_alloc(*b->b, x_dev, y_dev);
+  if (as_hip_stream_sync(b->b->main_stream) != 0) throw asx::Error(as_hip_last_error());
+  return 0;
+  AS_API_END(-1)
+}
+
+int64_t as_builder_static_scratch_need(as_builder *b) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b, "null builder");
+  return (int64_t)asx::static_scratch_need(*b->b);
+  AS_API_END(-1)
+}
+
 int as_builder_clears_y(as_builder *b) {
   AS_API_BEGIN
   AS_CHECK(b && b->b, "null builder");

@@ -257,6 +257,8 @@ void load_and_upload(Builder &b, int device) {
     b.x.bytes = b.cols * vs;
     HIPL(as_hip_alloc(&b.y.ptr, b.rows * vs));
     b.y.bytes = b.rows * vs;
+    // the static scratch array of this GPU, for the entry point that allocates nothing: looked up here, once
+    HIPL(as_hip_static_scratch(device, &b.static_scratch, &b.static_scratch_bytes));
     b.device_ready = true;
   }
   ensure_module(b);
@@ -275,15 +277,21 @@ void load_and_upload(Builder &b, int device) {
   }
 }
 
-// Launches the kernels of every active sub-matrix.
-static void launch_kernels(Builder &b, const void *x_dev, void *y_dev) {
+// Launches the kernels of every active sub-matrix.  static_scratch != nullptr: the kernels' scratch arrays are
+// 256-byte aligned pieces of that memory (in sub-matrix order) instead of the builder's own allocations.
+static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned char *static_scratch = nullptr) {
   size_t active = 0;
   auto skipped = [&](const SubKernel &k) { return !k.tpl || (b.only_sub >= 0 && &k != &b.subs[(size_t)b.only_sub]); };
   for (auto &k : b.subs) active += !skipped(k);
   bool multi = active > 1 && !b.serial_launch;
   if (multi) HIPL(as_hip_event_record(b.start_ev, b.main_stream));
+  uint64_t scratch_offset = 0;
   for (auto &k : b.subs) {
     void *scratch_ptr = k.scratch.ptr;
+    if (k.tpl && k.tpl->scratch_bytes && static_scratch) {
+      scratch_ptr = static_scratch + scratch_offset;
+      scratch_offset += (k.tpl->scratch_bytes + 255) / 256 * 256;
+    }
     if (skipped(k)) continue;
     AS_CHECK(k.uploaded && k.fn, "a template was changed after upload: call upload again");
     // kernel arguments: passed metadata arrays, val, col, x, y, scratch -- a fixed-size list, nothing allocated
@@ -347,6 +355,35 @@ void launch_spmv(Builder &b, const void *x_dev, void *y_dev) {
   check_launch_shapes(b);
   if (y_needs_clear(b)) zero_y(b, y_dev);
   launch_kernels(b, x_dev, y_dev);
+}
+
+uint64_t static_scratch_need(const Builder &b) {
+  uint64_t need = 0;
+  for (auto &k : b.subs)
+    if (k.tpl && k.tpl->scratch_bytes) need += (k.tpl->scratch_bytes + 255) / 256 * 256;
+  return need;
+}
+
+void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev) {
+  AS_CHECK(b.device_ready && b.module && !b.module_stale, "builder is not on the device: call upload first (this entry point loads nothing)");
+  for (auto &k : b.subs) AS_CHECK(!k.tpl || k.uploaded, "a template was changed after upload: call upload again");
+  check_launch_shapes(b);
+  const uint64_t need = static_scratch_need(b);
+  AS_CHECK(need <= b.static_scratch_bytes,
+           "the kernels of this graph need " + std::to_string(need) + " bytes of scratch, the static scratch array holds " +
+               std::to_string(b.static_scratch_bytes) + ": use as_builder_spmv_device");
+  AS_CHECK(need == 0 || b.static_scratch, "no static scratch array on this device");
+  unsigned char *base = (unsigned char *)b.static_scratch;
+  // Every call on this GPU shares the array, which holds what the last call left: the pieces whose kernels add
+  // into them are cleared by the fill kernel (no memset node, so the sequence can be captured)
+  uint64_t offset = 0;
+  for (auto &k : b.subs) {
+    if (!k.tpl || !k.tpl->scratch_bytes) continue;
+    if (k.tpl->scratch_starts_zero) zero_words(b, base + offset, (k.tpl->scratch_bytes + 3) / 4);
+    offset += (k.tpl->scratch_bytes + 255) / 256 * 256;
+  }
+  if (y_needs_clear(b)) zero_y(b, y_dev);
+  launch_kernels(b, x_dev, y_dev, base ? base : nullptr);
 }
 
 void spmv_host(Builder &b, const void *x_host, void *y_host) {

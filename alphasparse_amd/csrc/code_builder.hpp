@@ -36,6 +36,8 @@ struct Builder {
   void *zero_fn = nullptr;
   void *main_stream = nullptr, *start_ev = nullptr, *t0 = nullptr, *t1 = nullptr;
   DeviceBuf x, y;
+  void *static_scratch = nullptr;  // the library's static scratch array on this GPU (launch_spmv_no_alloc)
+  uint64_t static_scratch_bytes = 0;
   bool device_ready = false;
   bool module_stale = true;  // source changed since the module was loaded
   // false: every sub-matrix kernel runs on its own stream, all at once; true: one after the other on
@@ -71,6 +73,12 @@ void load_and_upload(Builder &b, int device);     // module load + arrays to HBM
 bool y_needs_clear(const Builder &b);
 // y = A x on device buffers already holding x; y is cleared first where y_needs_clear says so.
 void launch_spmv(Builder &b, const void *x_dev, void *y_dev);
+// The same SpMV for callers that must not allocate device memory: nothing is compiled, loaded or allocated
+// (the builder must be uploaded), and the kernels' scratch arrays are pieces of the library's static scratch
+// array on this GPU instead of the builder's own.  Fails when the graph needs more scratch than the array holds.
+// Calls that overlap on one GPU share the array and race.
+void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev);
+uint64_t static_scratch_need(const Builder &b);  // bytes of the static array the graph's kernels would use
 void spmv_host(Builder &b, const void *x_host, void *y_host);
 // Timing: `reps` launches of all kernels.  sync_each_launch reproduces the
 // upstream loop (kernel; cudaDeviceSynchronize, code_builder.cc:1524-1557).

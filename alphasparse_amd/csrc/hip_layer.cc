@@ -9,6 +9,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -25,9 +26,41 @@ static int fail(const std::string &what, const char *detail) {
     if (e_ != hipSuccess) return fail(#expr, hipGetErrorString(e_)); \
   } while (0)
 
+// Device memory that the library holds from its first upload on a GPU until the process ends, for the one entry
+// point that must not allocate (as_builder_spmv_device_no_alloc): the kernels' scratch arrays are carved out of
+// it instead of out of allocations of the builder.  Host code never uses the array's name as an address (on the
+// host it is only a stand-in for the symbol): as_hip_static_scratch asks the runtime for the address the array has
+// on the current GPU and hands that pointer out.  Every GPU has its own copy at its own address.
+// (No `used` attribute on it: with that attribute the compiler keeps the device-side symbol local to the code
+// object instead of exporting it for the host's lookup, and hipGetSymbolAddress cannot find it.)
+static __device__ __align__(256) unsigned char scratch[AS_STATIC_SCRATCH_BYTES];
+static const int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
 extern "C" {
 
 const char *as_hip_last_error(void) { return g_hip_err.c_str(); }
+
+// Address and size of the static scratch array on `device` (looked up once per device, with that device
+// current; later calls return the kept pointer and touch no HIP state).
+int as_hip_static_scratch(int device, void **ptr, uint64_t *bytes) {
+  if (device < 0 || device >= kMaxDevices || !ptr) return fail("as_hip_static_scratch", "bad device");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    int current = -1;
+    HIP_TRY(hipGetDevice(&current));
+    if (current != device) HIP_TRY(hipSetDevice(device));
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (current != device) (void)hipSetDevice(current);
+    if (e != hipSuccess || !p) return fail("hipGetSymbolAddress(scratch)", hipGetErrorString(e));
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  if (bytes) *bytes = AS_STATIC_SCRATCH_BYTES;
+  return 0;
+}
 
 int as_hip_device_count(void) {
   int n = 0;

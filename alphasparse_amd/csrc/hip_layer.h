@@ -9,6 +9,7 @@ extern "C" {
 const char *as_hip_last_error(void);
 int as_hip_device_count(void);
 int as_hip_init(int device);
+int as_hip_static_scratch(int device, void **ptr, uint64_t *bytes);
 int as_hip_device_info(int device, char *name, int name_cap, int *cu_count, int *wave_size, uint64_t *lds_per_block,
                        uint64_t *global_mem);
 int as_hip_compile(const char *src, const char *arch, const char *const *opts, int n_opts, void **code,

@@ -82,6 +82,9 @@ struct Template {
   // Device scratch of the kernels (last argument `scratch_arr`): allocated and cleared once at upload; what
   // it holds between two SpMVs is the template's business (the tile template leaves it cleared).  0 = none.
   uint64_t scratch_bytes = 0;
+  // true: the kernels rely on the scratch array holding zeros when an SpMV starts (the tile template adds row
+  // sums into it and clears it again); false: every word that is read was written earlier in the same SpMV
+  bool scratch_starts_zero = false;
   // > 0: a second kernel `spmv_<sub>_finish` with this many workgroups follows spmv_<sub> on the same
   // stream (same arguments)
   uint64_t finish_tblock_num = 0, finish_thread_num = 256, finish_lds_bytes = 0;

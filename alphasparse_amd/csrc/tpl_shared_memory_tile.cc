@@ -132,6 +132,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   // stores: the rows of a row strip belong to this kernel alone.
   if (t->global_sort_index && !sub_block_is_col_restricted(m, sub)) {
     t->scratch_bytes = sub_rows * vs;
+    t->scratch_starts_zero = true;  // row sums are added into it; the finish kernel leaves it cleared
     t->is_atom_add = false;  // y itself is written once, by the finish kernel
     t->finish_tblock_num = std::max<uint64_t>(1, std::min<uint64_t>(1024, (sub_rows + 255) / 256));
   }

@@ -255,6 +255,19 @@ int as_builder_spmv(as_builder *b, const void *x_host, void *y_host);
 int as_builder_spmv_device(as_builder *b, const void *x_dev, void *y_dev);
 /* 1 when an SpMV of the builder's current templates starts with a clear of y, 0 when it does not; <0 error */
 int as_builder_clears_y(as_builder *b);
+/* No counterpart in the reference.  as_builder_spmv_device for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the call compiles, loads and
+ * allocates nothing.  The builder must have been uploaded and not changed since (else an error), and the scratch
+ * arrays of its kernels (row sums of a sorted tile strip, the products of the product-bin template) are 256-byte
+ * aligned pieces of one static device array of AS_STATIC_SCRATCH_BYTES that the library holds on every GPU it has
+ * uploaded to, until the process ends.  A graph whose kernels need more scratch than that
+ * (as_builder_static_scratch_need) is rejected with an error: use as_builder_spmv_device for it.  All calls on
+ * one GPU share the array, which keeps what the last call left (the pieces that must start at zero are cleared
+ * by a fill kernel at the start of the call): calls that overlap on one GPU race. */
+#define AS_STATIC_SCRATCH_BYTES (64u << 20)
+int as_builder_spmv_device_no_alloc(as_builder *b, const void *x_dev, void *y_dev);
+/* bytes of the static scratch array the kernels of the builder's current templates would use (0: none) */
+int64_t as_builder_static_scratch_need(as_builder *b);
 /* 0 (default): the kernels of the sub-matrices run concurrently, one stream each (code_builder.cc:1517-1518);
  * 1: one after the other on the caller's stream.  No counterpart in the reference. */
 int as_builder_set_serial_launch(as_builder *b, int serial);
@@ -361,6 +374,9 @@ int64_t as_template_node_report(int template_type, long tblock_num, long thread_
 const char *as_hip_last_error(void);
 int as_hip_device_count(void);
 int as_hip_init(int device);                                   /* cudaSetDevice(DEFAULT_DEVICE_ID), code_builder.cc:1489 */
+/* no counterpart in the reference: address (on `device`) and size of the library's static scratch array, see
+ * as_builder_spmv_device_no_alloc; looked up once per device, later calls return the kept pointer */
+int as_hip_static_scratch(int device, void **ptr, uint64_t *bytes);
 int as_hip_device_info(int device, char *name, int name_cap, int *cu_count, int *wave_size, uint64_t *lds_per_block,
                        uint64_t *global_mem);
 /* hipRTC: HIP source -> gfx950 code object (malloc'ed, release with as_hip_free_host); needs no GPU */
