@@ -34,6 +34,9 @@ const char *dtype_c_name(DType t) {
 // get_matrix_index_and_val_from_file (struct.cc:92-175): first non-blank line is
 // "rows cols [nnz]", every further line "row col val", 1-based, rows
 // non-decreasing.  Lines starting with white space are skipped, as upstream.
+// Upstream takes whatever atol / stof make of a line (an index of 0 wraps to 2^64 - 1, an index beyond the header
+// is kept); here every entry is checked against the header and a line that does not parse is an error, because
+// the indices end up addressing x and y on the device.
 CooInput read_coo_file(const std::string &path, DType val_dtype) {
   AS_CHECK(val_dtype == FLOAT || val_dtype == DOUBLE, "value type must be FLOAT or DOUBLE");
   std::ifstream in(path, std::ios::binary);
@@ -42,25 +45,39 @@ CooInput read_coo_file(const std::string &path, DType val_dtype) {
   out.val_dtype = val_dtype;
   std::string line;
   bool first = true;
+  uint64_t line_no = 0;
   while (std::getline(in, line)) {
     if (line.empty() || isspace((unsigned char)line[0])) continue;
+    line_no++;
+    const std::string where = path + ", entry line " + std::to_string(line_no);
     const char *p = line.c_str();
     char *e = nullptr;
     long a = strtol(p, &e, 10);
-    long b = strtol(e, &e, 10);
+    AS_CHECK(e != p, "malformed line (no row index) in " + where);
+    const char *q = e;
+    long b = strtol(q, &e, 10);
+    AS_CHECK(e != q, "malformed line (no column index) in " + where);
     if (first) {
+      AS_CHECK(a > 0 && b > 0, "matrix sizes must be positive in " + path);
       out.row_index_max = (uint64_t)(a - 1);
       out.col_index_max = (uint64_t)(b - 1);
       first = false;
       continue;
     }
+    AS_CHECK(a >= 1 && (uint64_t)a <= out.row_index_max + 1, "row index outside 1..rows in " + where);
+    AS_CHECK(b >= 1 && (uint64_t)b <= out.col_index_max + 1, "column index outside 1..cols in " + where);
     uint64_t r = (uint64_t)(a - 1), c = (uint64_t)(b - 1);
     AS_CHECK(out.row.empty() || r >= out.row.back(), "row indices must be non-decreasing");
     out.row.push_back(r);
     out.col.push_back(c);
     // stof / stod semantics: the value is parsed at its own precision.
-    out.val.push_back(val_dtype == DOUBLE ? strtod(e, nullptr) : (double)strtof(e, nullptr));
+    q = e;
+    const double v = val_dtype == DOUBLE ? strtod(q, &e) : (double)strtof(q, &e);
+    AS_CHECK(e != q, "malformed line (no value) in " + where);
+    out.val.push_back(v);
   }
+  AS_CHECK(!first, "no header line in " + path);
+  AS_CHECK(!out.row.empty(), "no entries in " + path);
   return out;
 }
 
@@ -260,6 +277,9 @@ std::unique_ptr<Matrix> matrix_from_coo(const CooInput &in, unsigned wave) {
   AS_CHECK(in.val_dtype == FLOAT || in.val_dtype == DOUBLE, "value type must be FLOAT or DOUBLE");
   AS_CHECK(!in.row.empty() && in.row.size() == in.col.size() && in.row.size() == in.val.size(), "malformed COO");
   AS_CHECK(wave == 32 || wave == 64, "wave must be 32 or 64");
+  // every entry path ends here: no index may point outside x or y
+  for (size_t i = 0; i < in.row.size(); i++)
+    AS_CHECK(in.row[i] <= in.row_index_max && in.col[i] <= in.col_index_max, "entry " + std::to_string(i) + " lies outside the matrix");
   auto m = std::make_unique<Matrix>();
   m->rows = m->y_rows = in.row_index_max + 1;
   m->cols = in.col_index_max + 1;

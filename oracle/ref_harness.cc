@@ -47,6 +47,25 @@ extern "C" {
 // chdir to the directory holding the redirected global_config.json
 int ref_init(const char *config_dir) { return chdir(config_dir); }
 
+// The reference's own reader of .mtx.coo text (struct.cc:92-175).  Returns the number of entries; copies
+// min(nnz, cap) of them (0-based indices, values widened to double) and header = {max row index, max column index}.
+int64_t ref_read_coo_file(const char *path, int val_dtype, uint64_t *row, uint64_t *col, double *val, uint64_t cap,
+                          uint64_t header[2]) {
+  Quiet q;
+  vector<unsigned long> r, c;
+  vector<float> vf;
+  vector<double> vd;
+  unsigned long max_row = 0, max_col = 0;
+  get_matrix_index_and_val_from_file(path, r, c, vf, vd, (data_type)val_dtype, max_row, max_col);
+  for (uint64_t i = 0; i < r.size() && i < cap; i++) {
+    row[i] = r[i];
+    col[i] = c[i];
+    val[i] = val_dtype == FLOAT ? (double)vf[i] : vd[i];
+  }
+  if (header) { header[0] = max_row; header[1] = max_col; }
+  return (int64_t)r.size();
+}
+
 void *ref_matrix_from_coo(uint64_t rows, uint64_t cols, uint64_t nnz, const uint64_t *row, const uint64_t *col,
                           const double *val, int val_dtype) {
   Quiet q;

@@ -25,6 +25,8 @@ MATRICES = {
     "fem": (lambda: S.fem_blocks(30, 9, 12, seed=9), K.DOUBLE),
     "irr": (lambda: S.extreme_irregular(220, 3, 150, 219, seed=10), K.DOUBLE),
     "steps": (lambda: _steps([3] * 40 + [20] * 24 + [90] * 8, 128, 11), K.FLOAT),
+    # benchmark configuration 1 at its stated shape: 4096 x 4096, exactly 8 elements per row, fp32
+    "c1": (lambda: S.uniform_rows(), K.FLOAT),
 }
 
 D3 = [(K.DENSE_ROW_COARSE_SORT_FIXED, (1,)),
@@ -78,6 +80,9 @@ FORMAT_CASES = [
     ("finesort_irr_ell", "irr", FINE_SORT, "S5", {"wave": 32}),
     ("bandsort_pl_csr5", "pl", BAND_SORT, "S9", {"t": 3}),
     ("bandsort_irr_longrow", "irr", BAND_SORT, "S8", {"b": 32}),
+    # configuration 1 (4096 x 4096, 8 per row) through the ELL graph and through the SELL graph the search returns for it
+    ("c1_ell", "c1", [], "S5", {"wave": 32}),
+    ("c1_sell512", "c1", [], "S1", {"m": 512}),
 ]
 
 

@@ -137,3 +137,110 @@ def test_binary_cache_rejects_damaged_files(tmp_path):
     path.write_bytes(bytes(bad))
     with pytest.raises(A.AlphaSparseError):
         A.Matrix.from_binary_file(path)
+
+
+# ---- the .mtx.coo reader against a literal file and against the reference's own reader ------------------------------
+# 1-based indices, rows non-decreasing, header with and without the element count, values in the spellings stof /
+# stod accept, a blank line and a line that starts with white space (both skipped by the reference, struct.cc:121).
+COO_TEXT = """4 6 7
+1 1 4.0
+1 6 -1
+2 3 1.25E+2
+
+3 1 0.1
+ 9 9 9
+3 4 -8e-3
+4 2 1e-40
+4 6 16777217
+"""
+COO_KNOWN = dict(rows=4, cols=6, row=[0, 0, 1, 2, 2, 3, 3], col=[0, 5, 2, 0, 3, 1, 5],
+                 val=[4.0, -1.0, 125.0, 0.1, -8e-3, 1e-40, 16777217.0])
+
+
+@pytest.mark.parametrize("vdt,npd", [(K.FLOAT, np.float32), (K.DOUBLE, np.float64)], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("header", ["4 6 7", "4 6"], ids=["with_nnz", "without_nnz"])
+def test_coo_file_known_answer(tmp_path, vdt, npd, header):
+    p = tmp_path / "k.mtx.coo"
+    p.write_text(COO_TEXT.replace("4 6 7", header, 1))
+    m = A.Matrix.from_coo_file(p, vdt)
+    info = m.info()
+    assert (info["rows"], info["cols"], info["nnz"]) == (COO_KNOWN["rows"], COO_KNOWN["cols"], 7)
+    r, c, v = _coo(m)
+    assert r.tolist() == COO_KNOWN["row"] and c.tolist() == COO_KNOWN["col"]
+    # every value rounded once, from the decimal text to the value type (stof / stod): 0.1 and 16777217 differ
+    # between float and double, 1e-40 is a float denormal
+    want = np.array([npd(t) for t in ("4.0", "-1", "1.25E+2", "0.1", "-8e-3", "1e-40", "16777217")]).astype(np.float64)
+    assert np.array_equal(v, want)
+    assert m.check_sorted() and not m.has_empty_row()
+
+
+def _ref_read(path, vdt):
+    import ctypes as C
+    import ref_lib
+    L = ref_lib.lib()
+    L.ref_read_coo_file.restype = C.c_int64
+    L.ref_read_coo_file.argtypes = [C.c_char_p, C.c_int, K.u64p, K.u64p, K.f64p, C.c_uint64, K.u64p]
+    hdr = np.zeros(2, np.uint64)
+    n = L.ref_read_coo_file(str(path).encode(), vdt, None, None, None, 0, hdr.ctypes.data_as(K.u64p))
+    r, c, v = np.zeros(n, np.uint64), np.zeros(n, np.uint64), np.zeros(n, np.float64)
+    L.ref_read_coo_file(str(path).encode(), vdt, r.ctypes.data_as(K.u64p), c.ctypes.data_as(K.u64p), v.ctypes.data_as(K.f64p), n,
+                        hdr.ctypes.data_as(K.u64p))
+    return int(hdr[0]) + 1, int(hdr[1]) + 1, r.astype(np.int64), c.astype(np.int64), v
+
+
+def _needs_reference():
+    import ref_lib
+    if not ref_lib.available():
+        pytest.skip("oracle/_ref/libasref.so is not built (make -C oracle ref, needs the reference sources)")
+
+
+@pytest.mark.parametrize("where", ["cpu", pytest.param("gpu_box", marks=pytest.mark.gpu)])
+@pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
+def test_coo_file_reader_matches_the_reference_reader(tmp_path, vdt, where):
+    """as_matrix_from_coo_file against get_matrix_index_and_val_from_file (struct.cc:92-175) compiled from the
+    reference's own source: the literal file with and without the element count, and generated files whose values
+    are written with 9 and 17 significant digits, in plain and in exponent spelling."""
+    _needs_reference()
+    # (the reference's stof throws on a value that is no normal float, and the exception ends the process: the
+    # denormal of the literal file is only given to the fp64 reader, and generated values stay within float range)
+    literal = COO_TEXT if vdt == K.DOUBLE else COO_TEXT.replace("1e-40", "1e-30")
+    texts = [literal, literal.replace("4 6 7", "4 6", 1)]
+    rng = np.random.default_rng(11)
+    for seed, fmt in ((1, "%.9g"), (2, "%.17g"), (3, "%e"), (4, "%.3f")):
+        rows, cols, r, c, _, _ = cases._steps([3, 1, 40, 1, 5, 9, 2, 6, 1, 1] * 7, 900, seed)
+        vals = rng.standard_normal(len(r)) * 10.0 ** rng.integers(-25, 25, len(r))
+        lines = ["%d %d %d" % (rows, cols, len(r))] + ["%d %d %s" % (a + 1, b + 1, fmt % x) for a, b, x in zip(r, c, vals)]
+        texts.append("\n".join(lines) + ("\n" if seed % 2 else ""))          # with and without a final newline
+    for i, text in enumerate(texts):
+        p = tmp_path / ("m%d.mtx.coo" % i)
+        p.write_text(text)
+        m = A.Matrix.from_coo_file(p, vdt)
+        info = m.info()
+        r, c, v = _coo(m)
+        ref_rows, ref_cols, rr, rc, rv = _ref_read(p, vdt)
+        assert (info["rows"], info["cols"], info["nnz"]) == (ref_rows, ref_cols, len(rr)), i
+        assert np.array_equal(r, rr) and np.array_equal(c, rc), i
+        assert np.array_equal(v.view(np.uint64), rv.view(np.uint64)), i      # bit for bit
+
+
+@pytest.mark.parametrize("bad,why", [
+    ("3 3 2\n1 1 1\n0 2 1\n", "row index 0"), ("3 3 2\n1 0 1\n2 2 1\n", "column index 0"),
+    ("3 3 2\n1 1 1\n4 2 1\n", "row beyond the header"), ("3 3 2\n1 4 1\n2 2 1\n", "column beyond the header"),
+    ("3 3 2\n1 1 1\n2 2\n", "no value"), ("3 3 2\n1 1 1\nx 2 1\n", "row does not parse"),
+    ("3 3 2\n1 1 1\n2 y 1\n", "column does not parse"), ("3 3 2\n1 1 1\n2 2 z\n", "value does not parse"),
+    ("3 3 2\n2 1 1\n1 2 1\n", "rows decrease"), ("0 3 1\n1 1 1\n", "no rows"), ("3 3 0\n", "no entries"), ("", "empty file"),
+    ("3 3 2\n1 1 1\n-2 2 1\n", "negative row")], ids=lambda t: t.replace(" ", "_") if " " in t and "\n" not in t else None)
+def test_coo_file_rejects_bad_entries(tmp_path, bad, why):
+    """An entry outside the matrix would address x or y out of bounds on the device: the reader stops instead
+    (the reference takes whatever atol makes of the line: struct.cc:140-141)."""
+    p = tmp_path / "bad.mtx.coo"
+    p.write_text(bad)
+    with pytest.raises(A.AlphaSparseError):
+        A.Matrix.from_coo_file(p, K.FLOAT)
+
+
+def test_from_coo_arrays_rejects_entries_outside_the_matrix():
+    with pytest.raises(A.AlphaSparseError):
+        A.Matrix.from_coo(3, 3, [0, 3], [0, 1], np.ones(2), K.FLOAT)
+    with pytest.raises(A.AlphaSparseError):
+        A.Matrix.from_coo(3, 3, [0, 1], [0, 3], np.ones(2), K.FLOAT)

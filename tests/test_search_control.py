@@ -13,13 +13,18 @@ from alphasparse_amd import _capi as K
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "search_control.json")
 
 
+# no GPU needed: run in the CPU suite and once more, under the `gpu` marker, in the suite of the GPU box
+EVERYWHERE = pytest.mark.parametrize("where", ["cpu", pytest.param("gpu_box", marks=pytest.mark.gpu)])
+
+
 @pytest.fixture(scope="module")
 def want():
     with open(GOLDEN) as f:
         return json.load(f)
 
 
-def test_param_enumerator_matches_upstream(want):
+@EVERYWHERE
+def test_param_enumerator_matches_upstream(want, where):
     for case, w in zip(H.ENUM_CASES, want["enumerator"]):
         got = H.enumerate_params(K.lib(), "as_", *case)
         assert got.tolist() == w, case
@@ -30,7 +35,8 @@ def test_param_enumerator_is_an_odometer():
     assert got.tolist() == [[a, b] for b in (10, 20, 30) for a in (1, 2, 3)]   # knob 0 fastest
 
 
-def test_stop_rule_matches_upstream(want):
+@EVERYWHERE
+def test_stop_rule_matches_upstream(want, where):
     for (struggle, g), w in zip(H.STOP_CASES, want["stop_rule"]):
         assert H.stop_rule(K.lib(), "as_", struggle, g) == w, (struggle, g[:8])
 
@@ -44,12 +50,14 @@ def test_stop_rule_window_and_struggle_steps():
     assert go[:26] == [1] * 26 and go[26] == 0
 
 
-def test_strategy_report_matches_upstream(want):
+@EVERYWHERE
+def test_strategy_report_matches_upstream(want, where):
     for (s, p), w in zip(H.STRATEGY_CASES, want["strategy_report"]):
         assert H.strategy_report(K.lib(), "as_", s, p) == w
 
 
-def test_template_node_report_matches_upstream(want):
+@EVERYWHERE
+def test_template_node_report_matches_upstream(want, where):
     for case, w in zip(H.TEMPLATE_NODE_CASES, want["template_node_report"]):
         assert H.template_node_report(K.lib(), "as_", *case) == w, K.TEMPLATE_NAMES[case[0]]
 

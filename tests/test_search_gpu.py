@@ -65,6 +65,25 @@ def test_search_result_is_correct_and_reported(gpu, name):
     b.close()
 
 
+def test_configuration_1_at_its_stated_shape(gpu):
+    """Benchmark configuration 1 exactly as stated: 4096 x 4096, 8 elements in every row at seeded uniform columns
+    (32,768 elements), values and x in [-1, 1], fp32.  A short search, then the rebuilt best graph against the CPU
+    CSR oracle, with y full of NaN before the call as well."""
+    rows, cols, r, c, v, x = S.uniform_rows()
+    assert (rows, cols, len(r)) == (4096, 4096, 32768) and v.dtype == np.float32
+    assert np.all(np.bincount(np.asarray(r, np.int64), minlength=rows) == 8)
+    assert np.all(np.abs(v) <= 1) and np.all(np.abs(x) <= 1)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.FLOAT, wave=64)
+    res = A.find_best_graph(m, total_time_s=8.0, device=gpu, timed_region_ms=3.0)
+    print("C1 best %.1f GFLOP/s, %d candidates, %.1f s" % (res.gflops, res.candidates, res.seconds), flush=True)
+    assert res.gflops > 0 and res.candidates > 0 and res.failed_candidates == 0
+    b = _check_best(res, rows, r, c, v, x, gpu, np.float32)
+    y_ref, mag = _oracle(rows, r, c, v, x)
+    rel, ratio, tol = O.check_y(b.spmv_device(x), y_ref, mag, np.float32)
+    assert rel <= tol and ratio <= 1.0, (rel, ratio)
+    b.close()
+
+
 def _random_rows(rows, cols, per_row, seed):
     """rows x cols, per_row elements in every row at sorted random columns, fp values in [-1, 1)."""
     rng = np.random.default_rng(seed)
