@@ -159,9 +159,13 @@ struct Ctx {
   const SearchOptions &opt;
   SearchResult &res;
   SearchStrategy global;
-  std::vector<uint8_t> ones;  // x = 1 in the value type, `cols` entries
+  // the vector every candidate is checked (and timed) with, in the value type, `cols` entries: x[j] = 1 + j % 7.
+  // Not constant on purpose: a kernel that reads x at a wrong place (relative, diagonal and column-run column
+  // forms, x-slice offsets, the first column of a column band) gives a wrong y with it, which x = 1 would hide
+  std::vector<uint8_t> probe_x;
   bool empty_rows = false;    // the input has rows without elements and they are removed first
-  // per row of the input: the sum of its values = y for x = 1, and the sum of their magnitudes
+  // per row of the input: y for that x (a host CSR product computed once per search), and the same sum over the
+  // magnitudes
   std::vector<double> row_sum, row_mag;
   // time per SpMV (ms) of the best whole graph measured so far, 0 before the first: a strip kernel that alone takes
   // longer cannot be part of a better graph, whichever way the strips are launched
@@ -189,8 +193,8 @@ void set_launch(Template &t, const TemplateNode &n) {
 }
 
 // time the kernels of a builder: warm-up, a short probe, then ~timed_region_ms
-// One SpMV with x = 1: the rows that the loaded kernels cover (sub-matrix `sub`, or all with sub < 0) must
-// hold the sums of their values, every other row of y zero.  The bound is loose (1e-3 / 1e-9 of the sum of
+// One SpMV with the search's probe vector (x[j] = 1 + j % 7): the rows that the loaded kernels cover (sub-matrix
+// `sub`, or all with sub < 0) must hold the host's product for that x, every other row of y zero.  The bound is loose (1e-3 / 1e-9 of the sum of
 // the magnitudes): it is there to catch an element that was lost, doubled or added to the wrong row, not
 // rounding.  Throws on a mismatch.
 void verify_candidate(Ctx &c, Builder &b, const Matrix &m, int64_t sub) {
@@ -319,7 +323,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
       add_template_to_builder(*b, sub, type);
       compress_template_in_builder(*b, sub);
       load_and_upload(*b, c.opt.device);
-      if (as_hip_h2d(b->x.ptr, c.ones.data(), b->x.bytes) != 0) throw Error(as_hip_last_error());
+      if (as_hip_h2d(b->x.ptr, c.probe_x.data(), b->x.bytes) != 0) throw Error(as_hip_last_error());
     } catch (const std::exception &e) {
       c.res.failed_candidates++;
       c.log(std::string("  candidate failed: ") + e.what());
@@ -796,7 +800,7 @@ bool search_dense_strategy(Ctx &c, const CooInput &in, std::vector<StrategyNode>
   try {
     BuiltGraph bg = build_from_graph(in, out, c.opt.wave);
     load_and_upload(*bg.builder, c.opt.device);
-    if (as_hip_h2d(bg.builder->x.ptr, c.ones.data(), bg.builder->x.bytes) != 0) throw Error(as_hip_last_error());
+    if (as_hip_h2d(bg.builder->x.ptr, c.probe_x.data(), bg.builder->x.bytes) != 0) throw Error(as_hip_last_error());
     verify_candidate(c, *bg.builder, *bg.matrix, -1);
     time_builder(c, *bg.builder, out.time_ms, out.gflops);
     // kernels that each fill the machine can be faster one after the other than on concurrent streams
@@ -854,18 +858,19 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
   if (empty_rows) c.log("rows without elements are removed before the first operator of every graph");
   size_t cols = in.col_index_max + 1;
   if (in.val_dtype == DOUBLE) {
-    c.ones.resize(cols * 8);
-    for (size_t i = 0; i < cols; i++) ((double *)c.ones.data())[i] = 1.0;
+    c.probe_x.resize(cols * 8);
+    for (size_t i = 0; i < cols; i++) ((double *)c.probe_x.data())[i] = 1.0 + (double)(i % 7);
   } else {
-    c.ones.resize(cols * 4);
-    for (size_t i = 0; i < cols; i++) ((float *)c.ones.data())[i] = 1.0f;
+    c.probe_x.resize(cols * 4);
+    for (size_t i = 0; i < cols; i++) ((float *)c.probe_x.data())[i] = 1.0f + (float)(i % 7);
   }
   if (opt.verify_candidates) {
     c.row_sum.assign(in.row_index_max + 1, 0.0);
     c.row_mag.assign(in.row_index_max + 1, 0.0);
     for (size_t i = 0; i < in.row.size(); i++) {
-      c.row_sum[in.row[i]] += in.val[i];
-      c.row_mag[in.row[i]] += std::fabs(in.val[i]);
+      const double xj = 1.0 + (double)(in.col[i] % 7);
+      c.row_sum[in.row[i]] += in.val[i] * xj;
+      c.row_mag[in.row[i]] += std::fabs(in.val[i]) * xj;
     }
   }
   auto t_begin = std::chrono::steady_clock::now();
@@ -971,13 +976,13 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
     if (close.size() >= 2) {
       SearchOptions longer = opt;
       longer.timed_region_ms = opt.timed_region_ms * 4;
-      Ctx c2{longer, res, init_search_strategy(opt.struggle_step_num, 1e9), c.ones};
+      Ctx c2{longer, res, init_search_strategy(opt.struggle_step_num, 1e9), c.probe_x};
       float top = 0;
       for (BestGraph *g : close) {
         try {
           BuiltGraph bg = build_from_graph(in, *g, opt.wave);
           load_and_upload(*bg.builder, opt.device);
-          if (as_hip_h2d(bg.builder->x.ptr, c.ones.data(), bg.builder->x.bytes) != 0) throw Error(as_hip_last_error());
+          if (as_hip_h2d(bg.builder->x.ptr, c.probe_x.data(), bg.builder->x.bytes) != 0) throw Error(as_hip_last_error());
           time_builder(c2, *bg.builder, g->time_ms, g->gflops);
           c.log("final comparison " + g->dense_strategy_name + ": " + std::to_string(g->gflops) + " GFLOP/s" + c.stamp());
           if (g->gflops > top) { top = g->gflops; res.best = *g; res.seconds_to_best = g->found_at_s; }

@@ -97,7 +97,7 @@ struct SearchOptions {
   // true: the two general templates DIRECT_ATOM / SHARED_MEMORY, which upstream implements
   // (direct_atom_op.cc, shared_memory_op.cc) but keeps out of its white list, are searched as well
   bool general_templates = false;
-  // every candidate's y for x = 1 is compared with the sums of the rows' values before it is timed; a candidate
+  // every candidate's y for x[j] = 1 + j % 7 is compared with a host CSR product (computed once per search) before it is timed; a candidate
   // that differs counts as failed and cannot win
   bool verify_candidates = true;
 };

@@ -1,19 +1,28 @@
 #!/usr/bin/env python3
-"""Headline benchmark: SpMV GFLOP/s and fraction of the HBM roofline on one MI355X.
+"""Headline benchmark: SpMV GFLOP/s and fraction of the HBM roofline per matrix on one MI355X.
 
-A "step" is one y = A x over the whole matrix with every array already resident in HBM.  The workload
-is BASELINE configuration 2: the 5-point Laplacian on a 2048 x 2048 grid (4,194,304 rows, 20,963,328
-elements, fp32).  The operator graph and kernel are chosen by the search (tuning time is reported, not
-timed as steps); the result is verified against the CPU CSR oracle before anything is timed.
+A "step" is one y = A x over the whole matrix with every array already resident in HBM: exactly the launches
+the product call as_builder_spmv_device issues (the clear of y included where the graph needs it).  The
+headline workload is BASELINE configuration 2: the 5-point Laplacian on a 2048 x 2048 grid (4,194,304 rows,
+20,963,328 elements, fp32).  The operator graph and kernel are chosen by the search (tuning time is
+reported, not timed as steps); the result is verified against the CPU CSR oracle before anything is timed.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tune-seconds S] [--workload C1..C5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C1..C5] [--tune-seconds S] [--pin GRAPH]
 
-The other BASELINE configurations (C1 plumbing case, C3 power law, C4 FEM blocks, C5 extreme irregularity) run
-with --workload; with more than one row strip the roofline object is quoted on the strip kernel that takes
-the longest, timed alone, and "kernels" lists every strip kernel.
+Without --workload the line carries C2 as the headline (value, roofline, cpu_baseline) and `per_matrix`: one
+entry for each of the five BASELINE configurations (C1 plumbing case, C2 stencil, C3 power law, C4 FEM blocks,
+C5 extreme irregularity), each with its GFLOP/s, roofline fraction (also on the CSR floor), whole-SpMV fraction,
+tuning time, result check and CPU baseline.  C2, C5 and C1 are always searched; C3 and C4 are searched while the
+wall-clock budget (--budget-seconds) allows and otherwise run the committed winners of earlier searches
+(`tuning.mode` says which); a configuration that no longer fits the budget is recorded as skipped.
+With --workload only that configuration is measured and it is the headline.  With more than one row strip the
+roofline object is quoted on the strip kernel that takes the longest, timed alone, and "kernels" lists every
+strip kernel.
 
 Prints ONE JSON line (rank 0).  One GPU only: --gpus above 1 exits with a message."""
 import argparse
+import gc
+import hashlib
 import json
 import os
 import sys
@@ -24,9 +33,34 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+T_START = time.perf_counter()
+
+# name, generator, search budget (s) when measured alone / inside the five-matrix run, the committed winner of
+# earlier searches as a --pin graph, rough seconds for generation + format build + checks (budget planning)
+WORKLOADS = {
+    "C1": ("C1: 4096x4096 uniform, 8 per row, fp32", "uniform_rows", {}, 45.0, 6.0, "|S1:m=512@512", 5.0),
+    "C2": ("C2: 5-point Laplacian, 2048x2048 grid, 4194304 rows, fp32", "laplacian_5pt", {"grid": 2048}, 45.0, 30.0,
+           "S5,256,1,dia", 12.0),
+    "C3": ("C3: power-law row lengths (Zipf 1.8, mean 16, max 200000), 2000000 rows, uniform columns, fp32", "power_law",
+           {}, 90.0, 60.0, "sort+div64|T1@1024|T2:slice=8192,group=65536@512", 30.0),
+    "C4": ("C4: FEM-like dense 3x3 blocks, 27 block columns per block row in a +-2000 band, 1000002 rows, fp64",
+           "fem_blocks", {}, 45.0, 25.0, "|T1:slice=16384,group=4096@1024,runs", 35.0),
+    "C5": ("C5: 8000000 rows of 1-3 elements + 800 rows of 50000-1000000 elements, uniform columns, fp64",
+           "extreme_irregular", {"target_nnz": 60_000_000}, 150.0, 75.0,
+           "sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256", 45.0),
+}
+# the rocprofv3 summary that covers each configuration's kernels
+PROFILE_OF = {"C2": "profiles/spmv_ell_c2_laplacian_hbm_traffic.txt", "C3": "profiles/spmv_tile_product_bin_c3_power_law.txt",
+              "C4": "profiles/spmv_tile_c4_fem_blocks.txt", "C5": "profiles/spmv_tile_product_bin_c5_extreme_irregular.txt"}
+# HBM bytes per launch of the kernel the roofline object is quoted on, measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE (two runs, each scaled by what the same counter reads for the plain copy kernel of
+# --copy-calibration).  Keyed by the first 16 hex digits of the SHA-256 of the generated module source: a graph
+# whose kernels changed in any way since it was profiled reports null and names the profile instead.
+MEASURED_TRAFFIC = {
+}
 
 
-def cpu_baseline(rows, r, c, v, x, nnz):
+def cpu_baseline(rows, r, c, v, x, nnz, seconds):
     """The CPU CSR SpMV oracle (own restatement of the merge-path OpenMP baseline) on this host's cores."""
     import numpy as np
     import spmv_oracle as O
@@ -36,7 +70,7 @@ def cpu_baseline(rows, r, c, v, x, nnz):
     for _ in range(3):
         O.spmv_csr_merge(rp, ci, v, x, threads=threads)
     times = []
-    t_end = time.perf_counter() + 15.0
+    t_end = time.perf_counter() + seconds
     while len(times) < 10 or (time.perf_counter() < t_end and len(times) < 200):
         t0 = time.perf_counter()
         O.spmv_csr_merge(rp, ci, v, x, threads=threads)
@@ -46,32 +80,205 @@ def cpu_baseline(rows, r, c, v, x, nnz):
             "sample": "same matrix and x, OpenMP merge-path CSR, median of %d runs after 3 warm-ups" % len(times)}
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the
-# same counter reads for the plain copy kernel of --copy-calibration: x2.000 and x1.000); the summaries with the
-# full commands are under profiles/.  Keyed by what fixes the traffic of a launch:
-# workload, kernel template, rows per lane and the format's algorithmic bytes.  The thread count of the
-# workgroup changes neither the arrays read nor the lines written, so it is not part of the key.
-MEASURED_TRAFFIC = {
-    # profiles/spmv_ell_c2_laplacian_hbm_traffic.txt: diagonal form (what the search returns), 16-bit relative
-    # columns, 32-bit columns
-    ("C2", "DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS", 1, 117440514): 100803584 + 16777216,
-    ("C2", "DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS", 1, 159383552): 142747648 + 16777216,
-    ("C2", "DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS", 1, 201326592): 184690688 + 16777216,
-    # profiles/spmv_tile_product_bin_c3_power_law.txt: spmv_0 of the graph sort + two strips at row length 64
-    ("C3", "SHARED_MEMORY_TILE_TEMPLATE", 1, 188428272): 189857178 + 6688461,
-    # profiles/spmv_tile_c4_fem_blocks.txt: the tile kernel on the whole matrix, in its column-run form (what the
-    # search returns) and with 16-bit columns
-    ("C4", "SHARED_MEMORY_TILE_TEMPLATE", 1, 811515784): 802020352 + 13931827,
-    ("C4", "SHARED_MEMORY_TILE_TEMPLATE", 1, 882493768): 868082893 + 13931827,
-    # profiles/spmv_tile_product_bin_c5_extreme_irregular.txt: both passes of spmv_1 (sort + two strips at 16)
-    ("C5", "SHARED_MEMORY_PRODUCT_BIN_TEMPLATE", 1, 682067272): 288932454 + 132664525 + 197647974 + 79205786,
-}
+class _Pinned:
+    report, dense_strategy, n_sub, seconds_to_best, candidates, failed_candidates = "", 1, 1, 0.0, 0, 0
 
 
-def measured_traffic(workload, template, launch, algorithmic_bytes):
-    """HBM bytes per launch of the kernel the roofline object is quoted on, when that kernel was profiled."""
-    key = (workload.split(":")[0], template, int(launch["vec_width"]), int(algorithmic_bytes))
-    return MEASURED_TRAFFIC.get(key)
+def build_pinned(m, pin):
+    """A fixed graph instead of the search: 'S5,128,1[,rel|dia]' (one strip: skeleton, threads, rows per lane) or
+    'sort+div16|T1@1024|S1:m=128@128' (dense operators | one skeleton per strip, kernels one after the other)."""
+    import alphasparse_amd as A
+    from alphasparse_amd import _capi as K, skeletons as SK
+    res = _Pinned()
+    if "|" not in pin:
+        skel, threads, vec, *more = pin.split(",")
+        m.execute_strategy(K.COMPRESS_NONE)
+        templates = SK.apply_skeleton(m, 0, skel)
+        b = A.Builder(m)
+        b.set_template(0, templates[0])
+        if "rel" in more and not b.set_relative_columns(0):
+            raise SystemExit("bench.py: relative columns do not apply to this graph")
+        if "dia" in more and not b.set_diagonal_columns(0):
+            raise SystemExit("bench.py: diagonal columns do not apply to this graph")
+        b.set_launch(0, thread_num_in_block=int(threads), vec_width=int(vec))
+        return b, res
+    dense, *strips = pin.split("|")
+    for op in filter(None, dense.split("+")):
+        if op == "sort":
+            m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+            res.dense_strategy = 3
+        elif op.startswith("div"):
+            low = int(op[3:])
+            m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (low, low, 2, 0))
+            res.dense_strategy = max(res.dense_strategy, 2)
+        else:
+            raise SystemExit("bench.py: unknown dense operator %r in --pin" % op)
+    m.execute_strategy(K.COMPRESS_NONE)
+    res.n_sub = m.info()["n_sub"]
+    if len(strips) != res.n_sub:
+        raise SystemExit("bench.py: --pin names %d strips, the matrix has %d" % (len(strips), res.n_sub))
+    chosen = []
+    for s, spec in enumerate(strips):
+        spec, _, launch = spec.partition("@")
+        skel, _, kw = spec.partition(":")
+        kw = {k: int(x) for k, x in (p.split("=") for p in filter(None, kw.split(",")))}
+        words = [x for x in launch.split(",") if x]
+        chosen.append((SK.apply_skeleton(m, s, skel, **kw)[0], [int(x) for x in words if x.isdigit()], "runs" in words))
+    b = A.Builder(m)
+    for s, (tp, launch, runs) in enumerate(chosen):
+        b.set_template(s, tp)
+        if runs and not b.set_column_runs(s):
+            raise SystemExit("bench.py: the column-run form does not apply to strip %d" % s)
+        if launch:
+            b.set_launch(s, thread_num_in_block=launch[0], vec_width=launch[1] if len(launch) > 1 else 0)
+    b.set_serial_launch(True)
+    return b, res
+
+
+def measure(key, steps, warmup, tune_seconds, pin, cpu_seconds, copy_calibration=False, echo_report=False):
+    """One configuration end to end: generate, search (or pinned graph), check against the oracle, time.
+    Returns the full result object of that configuration."""
+    import numpy as np
+    import alphasparse_amd as A
+    from alphasparse_amd import _capi as K, synthetic as S
+    import spmv_oracle as O
+
+    name, gen, gen_kw, _, _, _, _ = WORKLOADS[key]
+    t_gen = time.perf_counter()
+    rows, cols, r, c, v, x = getattr(S, gen)(**gen_kw)
+    nnz = len(r)
+    val_dtype = K.DOUBLE if v.dtype == np.float64 else K.FLOAT
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), val_dtype, wave=64)
+    gen_s = time.perf_counter() - t_gen
+
+    t0 = time.perf_counter()
+    if pin:
+        b, res = build_pinned(m, pin)
+    else:
+        res = A.find_best_graph(m, total_time_s=tune_seconds, device=0)
+        b = res.build_best()
+    tune_s = time.perf_counter() - t0
+    b.compile().upload(0)
+    if echo_report and res.report:
+        print(res.report, file=sys.stderr)   # the best operator graph, as the search reports it
+
+    # correctness gate before any timing
+    y = b.spmv(x)
+    y_ref, mag = O.spmv_csr(O.coo_to_csr(rows, r), c.astype(np.uint32), v, x)
+    rel, ratio, tol = O.check_y(y, y_ref, mag, v.dtype.type)
+    if not (rel <= tol and ratio <= 1.0):
+        raise RuntimeError("%s: result check failed (rel L2 %.3e, per-row ratio %.2f)" % (key, rel, ratio))
+    del y, y_ref, mag
+
+    L = K.lib()
+    copy_gbs = None
+    if copy_calibration:
+        import ctypes as C
+        L.as_selftest_copy.argtypes = [C.c_int, C.c_uint64, C.c_int, C.POINTER(C.c_float)]
+        ms = C.c_float(0)
+        K.check(L.as_selftest_copy(0, 256 << 20, 20, C.byref(ms)), L)
+        copy_gbs = 2.0 * (256 << 20) / (ms.value * 1e-3) / 1e9
+    b.set_x(x)
+    b.time(max(1, warmup))                 # W untimed steps
+    L.as_hip_device_sync()
+    t0 = time.perf_counter()
+    kernel_ms, _ = b.time(steps)           # exactly K steps, events on the launch stream inside
+    L.as_hip_device_sync()
+    wall = time.perf_counter() - t0
+    gflops = 2.0 * nnz * steps / wall / 1e9
+    bytes_per_step = b.algorithmic_bytes()
+    per_launch_s = kernel_ms * 1e-3 / steps
+    achieved = bytes_per_step / per_launch_s / 1e9
+    # every strip kernel alone (events on its launch stream): algorithmic bytes = its format arrays + x once +
+    # the y rows of its strip (twice when it accumulates atomically into the cleared y)
+    vs = v.dtype.itemsize
+    reps = max(50, steps // 4)
+    kernels = []
+    for s in range(int(res.n_sub)):
+        ms, fmt_bytes, strip_rows, atom = b.time_sub_matrix(s, reps)
+        us = ms * 1e3 / reps
+        kb = fmt_bytes + cols * vs + strip_rows * vs * (2 if atom else 1)
+        kernels.append({"sub_matrix": s, "kernel_us": round(us, 3), "algorithmic_bytes": kb,
+                        "achieved_gbs": round(kb / us / 1e3, 1), "strip_rows": strip_rows})
+        try:  # templates with two kernels: each launched alone
+            kernels[-1]["pass_us"] = [round(b.time_sub_matrix_pass(s, which, reps) * 1e3 / reps, 3) for which in (1, 2)]
+        except A.AlphaSparseError:
+            pass
+    dominant = max(kernels, key=lambda k: k["kernel_us"])
+    if len(kernels) > 1:
+        achieved, roof_us, roof_bytes = dominant["achieved_gbs"], dominant["kernel_us"], dominant["algorithmic_bytes"]
+    else:
+        roof_us, roof_bytes = per_launch_s * 1e6, bytes_per_step
+    csr_floor = nnz * (v.dtype.itemsize + 4) + (rows + 1) * 4 + (rows + cols) * v.dtype.itemsize
+    sync_ok, sync_ms, sync_gf = A.part_execute_code_builder(b, [], 200)
+
+    templates = [b.describe(s)["template"] for s in range(int(res.n_sub))]
+    launches = [b.get_launch(s) for s in range(int(res.n_sub))]
+    source = b.kernel_source()
+    graph_hash = hashlib.sha256(source.encode()).hexdigest()[:16]
+
+    def column_form(sub):  # how the template of this sub-matrix stores its columns
+        d = b.describe(sub)
+        if any(k.startswith("diagonal_offset_") for k in d):
+            return "diagonal (computed, no array)"
+        if "col_run_mask" in d["arrays"]:
+            return "runs of consecutive columns"
+        if d["template"] == "DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS" and d["arrays"]["col_index_arr"][0] == "UNSIGNED_SHORT" \
+                and "(short)" in source:
+            return "16-bit relative"
+        return "explicit"
+    whole_gbs = bytes_per_step / per_launch_s / 1e9
+    out = {
+        "metric": "SpMV GFLOP/s and % of HBM BW roofline per matrix, 1xMI355X",
+        "value": round(gflops, 2), "unit": "GFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(wall * 1e3 / steps, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64" if v.dtype == np.float64 else "f32", "data": "synthetic",
+        "config": {"workload": name, "rows": rows, "nnz": nnz, "pinned": pin,
+                   "dense_strategy": int(res.dense_strategy), "sub_matrices": int(res.n_sub),
+                   "template": templates, "launch": launches,
+                   "columns": [column_form(s) for s in range(int(res.n_sub))],
+                   "clears_y": b.clears_y(), "graph_hash": graph_hash},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(graph_hash), "traffic_profile": PROFILE_OF.get(key),
+                     "kernel_us": round(roof_us, 3), "algorithmic_bytes": roof_bytes,
+                     "kernel": "spmv_%d (%s)" % (dominant["sub_matrix"], templates[dominant["sub_matrix"]]),
+                     "csr_floor_bytes": csr_floor,
+                     "csr_floor_frac": round(csr_floor / per_launch_s / 1e9 / HBM_PEAK_GBS, 4)},
+        "whole_spmv": {"us": round(per_launch_s * 1e6, 3), "algorithmic_bytes": bytes_per_step,
+                       "achieved_gbs": round(whole_gbs, 1), "frac": round(whole_gbs / HBM_PEAK_GBS, 4),
+                       "kernel_gflops": round(2.0 * nnz / per_launch_s / 1e9, 2)},
+        "kernels": kernels,
+        "tuning": {"mode": "pinned" if pin else "search", "seconds": round(tune_s, 2),
+                   "seconds_to_best": round(res.seconds_to_best, 2),
+                   "candidates": int(res.candidates), "failed": int(res.failed_candidates),
+                   "generation_seconds": round(gen_s, 2)},
+        "per_launch_sync_gflops": round(sync_gf, 2) if sync_ok else None,
+        "check": {"rel_l2": float("%.3e" % rel), "per_row_bound_ratio": round(ratio, 4)},
+    }
+    if copy_gbs is not None:
+        out["copy_kernel_gbs"] = round(copy_gbs, 1)
+    b.close()
+    del b, res, m
+    if cpu_seconds > 0:
+        out["cpu_baseline"] = cpu_baseline(rows, r, c, v, x, nnz, cpu_seconds)
+    del r, c, v, x
+    gc.collect()
+    return out
+
+
+def per_matrix_entry(key, full):
+    """The part of a configuration's result that the per_matrix list carries."""
+    e = {"workload": key, "gflops": full["value"], "ms_per_step": full["ms_per_step"], "steps": full["steps"],
+         "dtype": full["dtype"], "rows": full["config"]["rows"], "nnz": full["config"]["nnz"],
+         "graph": {k: full["config"][k] for k in ("dense_strategy", "sub_matrices", "template", "launch", "columns",
+                                                   "clears_y", "graph_hash", "pinned")},
+         "roofline": {k: full["roofline"][k] for k in ("frac", "achieved", "kernel", "kernel_us", "algorithmic_bytes",
+                                                       "csr_floor_bytes", "csr_floor_frac", "traffic", "traffic_profile")},
+         "whole_spmv": full["whole_spmv"], "kernels": full["kernels"], "tuning": full["tuning"], "check": full["check"]}
+    if "cpu_baseline" in full:
+        e["cpu_baseline"] = full["cpu_baseline"]
+    return e
 
 
 def main():
@@ -80,10 +287,15 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--tune-seconds", type=float, default=None,
-                    help="search budget; default 45 s (C1, C2, C4), 90 s (C3), 150 s (C5)")
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+                    help="search budget; with --workload the default is 45 s (C1, C2, C4), 90 s (C3), 150 s (C5); in the "
+                         "five-matrix run 6 / 30 / 60 / 25 / 75 s for C1..C5")
+    ap.add_argument("--workload", default=None, choices=["C1", "C2", "C3", "C4", "C5"],
+                    help="measure this configuration only (default: all five, C2 as the headline)")
+    ap.add_argument("--budget-seconds", type=float, default=420.0,
+                    help="five-matrix run: wall-clock budget of the whole program; C3 / C4 fall back to their committed "
+                         "winners and a configuration is skipped when the budget would be exceeded")
     ap.add_argument("--pin", default=None, metavar="SKELETON,THREADS,VEC | DENSE|STRIP0|STRIP1...",
-                    help="skip the search and run a fixed graph: S5,128,1 (ELL, 128 threads, 1 row per lane; S5,128,1,rel with 16-bit relative columns), or with "
+                    help="with --workload: skip the search and run a fixed graph: S5,128,1 (ELL, 128 threads, 1 row per lane; S5,128,1,rel with 16-bit relative columns), or with "
                          "row strips 'sort+div16|T1@1024|S1:m=128@128' = coarse sort, two strips at row length 16, strip 0 "
                          "skeleton T1 with 1024 threads, strip 1 skeleton S1 (m = 128) with 128 threads, kernels one after "
                          "the other ('@1024,runs': the tile template in its column-run form); used for profiling runs that must all "
@@ -97,184 +309,58 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (rows would shard across GPUs with x "
               "replicated; see DESIGN.md).  Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.pin and not args.workload:
+        print("bench.py: --pin needs --workload", file=sys.stderr)
+        sys.exit(2)
 
-    import numpy as np
     import alphasparse_amd as A
-    from alphasparse_amd import _capi as K, synthetic as S
-    import spmv_oracle as O
-
     if A.device_count() < 1:
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
 
-    name, make = {
-        "C1": ("C1: 4096x4096 uniform, 8 per row, fp32", S.uniform_rows),
-        "C2": ("C2: 5-point Laplacian, 2048x2048 grid, 4194304 rows, fp32", lambda: S.laplacian_5pt(2048)),
-        "C3": ("C3: power-law row lengths (Zipf 1.8, mean 16, max 200000), 2000000 rows, uniform columns, fp32", S.power_law),
-        "C4": ("C4: FEM-like dense 3x3 blocks, 27 block columns per block row in a +-2000 band, 1000002 rows, fp64",
-               S.fem_blocks),
-        "C5": ("C5: 8000000 rows of 1-3 elements + 800 rows of 50000-1000000 elements, uniform columns, fp64",
-               lambda: S.extreme_irregular(target_nnz=60_000_000)),
-    }[args.workload]
-    if args.tune_seconds is None:
-        args.tune_seconds = {"C3": 90.0, "C5": 150.0}.get(args.workload, 45.0)
-    rows, cols, r, c, v, x = make()
-    nnz = len(r)
-    val_dtype = K.DOUBLE if v.dtype == np.float64 else K.FLOAT
-    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), val_dtype, wave=64)
+    if args.workload:
+        tune = args.tune_seconds if args.tune_seconds is not None else WORKLOADS[args.workload][3]
+        try:
+            out = measure(args.workload, args.steps, args.warmup, tune, args.pin, 0 if args.no_cpu_baseline else 15.0,
+                          args.copy_calibration, echo_report=True)
+        except RuntimeError as e:
+            print("bench.py: %s" % e, file=sys.stderr)
+            sys.exit(1)
+        print(json.dumps(out))
+        return
 
-    t0 = time.perf_counter()
-    if args.pin:
-        from alphasparse_amd import skeletons as SK
-
-        class _Pinned:
-            report, dense_strategy, n_sub, seconds_to_best, candidates, failed_candidates = "", 1, 1, 0.0, 0, 0
-        res = _Pinned()
-        if "|" not in args.pin:
-            skel, threads, vec, *more = args.pin.split(",")
-            m.execute_strategy(K.COMPRESS_NONE)
-            templates = SK.apply_skeleton(m, 0, skel)
-            b = A.Builder(m)
-            b.set_template(0, templates[0])
-            if "rel" in more and not b.set_relative_columns(0):
-                raise SystemExit("bench.py: relative columns do not apply to this graph")
-            if "dia" in more and not b.set_diagonal_columns(0):
-                raise SystemExit("bench.py: diagonal columns do not apply to this graph")
-            b.set_launch(0, thread_num_in_block=int(threads), vec_width=int(vec))
-        else:
-            dense, *strips = args.pin.split("|")
-            for op in filter(None, dense.split("+")):
-                if op == "sort":
-                    m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
-                    res.dense_strategy = 3
-                elif op.startswith("div"):
-                    low = int(op[3:])
-                    m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (low, low, 2, 0))
-                    res.dense_strategy = max(res.dense_strategy, 2)
-                else:
-                    raise SystemExit("bench.py: unknown dense operator %r in --pin" % op)
-            m.execute_strategy(K.COMPRESS_NONE)
-            res.n_sub = m.info()["n_sub"]
-            if len(strips) != res.n_sub:
-                raise SystemExit("bench.py: --pin names %d strips, the matrix has %d" % (len(strips), res.n_sub))
-            chosen = []
-            for s, spec in enumerate(strips):
-                spec, _, launch = spec.partition("@")
-                skel, _, kw = spec.partition(":")
-                kw = {k: int(x) for k, x in (p.split("=") for p in filter(None, kw.split(",")))}
-                words = [x for x in launch.split(",") if x]
-                chosen.append((SK.apply_skeleton(m, s, skel, **kw)[0], [int(x) for x in words if x.isdigit()], "runs" in words))
-            b = A.Builder(m)
-            for s, (tp, launch, runs) in enumerate(chosen):
-                b.set_template(s, tp)
-                if runs and not b.set_column_runs(s):
-                    raise SystemExit("bench.py: the column-run form does not apply to strip %d" % s)
-                if launch:
-                    b.set_launch(s, thread_num_in_block=launch[0], vec_width=launch[1] if len(launch) > 1 else 0)
-            b.set_serial_launch(True)
-    else:
-        res = A.find_best_graph(m, total_time_s=args.tune_seconds, device=0)
-        b = res.build_best()
-    tune_s = time.perf_counter() - t0
-    b.compile().upload(0)
-    if res.report:
-        print(res.report, file=sys.stderr)   # the best operator graph, as the search reports it
-
-    # correctness gate before any timing
-    y = b.spmv(x)
-    y_ref, mag = O.spmv_csr(O.coo_to_csr(rows, r), c.astype(np.uint32), v, x)
-    rel, ratio, tol = O.check_y(y, y_ref, mag, v.dtype.type)
-    if not (rel <= tol and ratio <= 1.0):
-        print("bench.py: result check failed (rel L2 %.3e, per-row ratio %.2f)" % (rel, ratio), file=sys.stderr)
-        sys.exit(1)
-
-    L = K.lib()
-    copy_gbs = None
-    if args.copy_calibration:
-        import ctypes as C
-        L.as_selftest_copy.argtypes = [C.c_int, C.c_uint64, C.c_int, C.POINTER(C.c_float)]
-        ms = C.c_float(0)
-        K.check(L.as_selftest_copy(0, 256 << 20, 20, C.byref(ms)), L)
-        copy_gbs = 2.0 * (256 << 20) / (ms.value * 1e-3) / 1e9
-    b.set_x(x)
-    b.time(max(1, args.warmup))                 # W untimed steps
-    L.as_hip_device_sync()
-    t0 = time.perf_counter()
-    kernel_ms, _ = b.time(args.steps)           # exactly K steps, events on the launch stream inside
-    L.as_hip_device_sync()
-    wall = time.perf_counter() - t0
-    gflops = 2.0 * nnz * args.steps / wall / 1e9
-    bytes_per_step = b.algorithmic_bytes()
-    per_launch_s = kernel_ms * 1e-3 / args.steps
-    achieved = bytes_per_step / per_launch_s / 1e9
-    # every strip kernel alone (events on its launch stream): algorithmic bytes = its format arrays + x once +
-    # the y rows of its strip (twice when it accumulates atomically into the cleared y)
-    vs = v.dtype.itemsize
-    kernels = []
-    for s in range(int(res.n_sub)):
-        ms, fmt_bytes, strip_rows, atom = b.time_sub_matrix(s, max(20, args.steps // 4))
-        us = ms * 1e3 / max(20, args.steps // 4)
-        kb = fmt_bytes + cols * vs + strip_rows * vs * (2 if atom else 1)
-        kernels.append({"sub_matrix": s, "kernel_us": round(us, 3), "algorithmic_bytes": kb,
-                        "achieved_gbs": round(kb / us / 1e3, 1), "strip_rows": strip_rows})
-        try:  # templates with two kernels: each launched alone
-            reps = max(20, args.steps // 4)
-            kernels[-1]["pass_us"] = [round(b.time_sub_matrix_pass(s, which, reps) * 1e3 / reps, 3) for which in (1, 2)]
-        except A.AlphaSparseError:
-            pass
-    dominant = max(kernels, key=lambda k: k["kernel_us"])
-    if len(kernels) > 1:
-        achieved, roof_us, roof_bytes = dominant["achieved_gbs"], dominant["kernel_us"], dominant["algorithmic_bytes"]
-    else:
-        roof_us, roof_bytes = per_launch_s * 1e6, bytes_per_step
-    csr_floor = nnz * (v.dtype.itemsize + 4) + (rows + 1) * 4 + (rows + cols) * v.dtype.itemsize
-    sync_ok, sync_ms, sync_gf = A.part_execute_code_builder(b, [], 200)
-
-    templates = [ln.split("=")[1] for s in range(int(res.n_sub))
-                 for ln in [b._L.as_template_describe(b._h, s).decode().splitlines()[0]]]
-    launches = [b.get_launch(s) for s in range(int(res.n_sub))]
-
-    def column_form(sub):  # how the ELL template of this sub-matrix stores its columns
-        d = b.describe(sub)
-        if any(k.startswith("diagonal_offset_") for k in d):
-            return "diagonal (computed, no array)"
-        if "col_run_mask" in d["arrays"]:
-            return "runs of consecutive columns"
-        if d["template"] == "DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS" and d["arrays"]["col_index_arr"][0] == "UNSIGNED_SHORT" \
-                and "(short)" in b.kernel_source():
-            return "16-bit relative"
-        return "explicit"
-    out = {
-        "metric": "SpMV GFLOP/s and % of HBM BW roofline per matrix, 1xMI355X",
-        "value": round(gflops, 2), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(wall * 1e3 / args.steps, 6), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f64" if v.dtype == np.float64 else "f32", "data": "synthetic",
-        "config": {"workload": name, "rows": rows, "nnz": nnz, "pinned": args.pin,
-                   "dense_strategy": int(res.dense_strategy), "sub_matrices": int(res.n_sub),
-                   "template": templates, "launch": launches,
-                   "columns": [column_form(s) for s in range(int(res.n_sub))]},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic(name, templates[dominant["sub_matrix"]], launches[dominant["sub_matrix"]],
-                                                 roof_bytes),
-                     "kernel_us": round(roof_us, 3), "algorithmic_bytes": roof_bytes,
-                     "kernel": "spmv_%d (%s)" % (dominant["sub_matrix"], templates[dominant["sub_matrix"]]),
-                     "csr_floor_bytes": csr_floor},
-        "whole_spmv": {"us": round(per_launch_s * 1e6, 3), "algorithmic_bytes": bytes_per_step,
-                       "achieved_gbs": round(bytes_per_step / per_launch_s / 1e9, 1),
-                       "frac": round(bytes_per_step / per_launch_s / 1e9 / HBM_PEAK_GBS, 4)},
-        "kernels": kernels,
-        "tuning": {"seconds": round(tune_s, 2), "seconds_to_best": round(res.seconds_to_best, 2),
-                   "candidates": int(res.candidates), "failed": int(res.failed_candidates)},
-        "per_launch_sync_gflops": round(sync_gf, 2) if sync_ok else None,
-        "check": {"rel_l2": float("%.3e" % rel), "per_row_bound_ratio": round(ratio, 4)},
-    }
-    if copy_gbs is not None:
-        out["copy_kernel_gbs"] = round(copy_gbs, 1)
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(rows, r, c, v, x, nnz)
+    # ---- all five configurations: C2 first (the headline), then the one whose search the configuration demands ----
+    results = {}
+    pm_steps = max(args.steps, 200)   # the other matrices: enough launches for a steady rate
+    for key in ("C2", "C5", "C3", "C4", "C1"):
+        _, _, _, _, tune_all, pinned, fixed_s = WORKLOADS[key]
+        tune = args.tune_seconds if args.tune_seconds is not None else tune_all
+        cpu_s = 0 if args.no_cpu_baseline else (15.0 if key == "C2" else 5.0)
+        left = args.budget_seconds - (time.perf_counter() - T_START)
+        pin = None
+        if key in ("C3", "C4") and left < fixed_s + tune + cpu_s + 15.0:
+            pin = pinned          # no room for a search: the committed winner
+        if key != "C2" and left < fixed_s + cpu_s + (0 if pin else tune):
+            results[key] = {"workload": key, "skipped": "budget",
+                            "seconds_left": round(left, 1)}
+            continue
+        print("[bench] %s: %s, %.0f s of budget left" % (key, "pinned graph" if pin else "search %.0f s" % tune, left),
+              file=sys.stderr, flush=True)
+        try:
+            full = measure(key, args.steps if key == "C2" else pm_steps, args.warmup, tune, pin, cpu_s,
+                           echo_report=(key == "C2"))
+        except RuntimeError as e:
+            if key == "C2":
+                print("bench.py: %s" % e, file=sys.stderr)
+                sys.exit(1)
+            results[key] = {"workload": key, "failed": str(e)}
+            continue
+        results[key] = full
+    out = dict(results["C2"])
+    out["per_matrix"] = [per_matrix_entry(k, results[k]) if "value" in results[k] else results[k]
+                         for k in ("C1", "C2", "C3", "C4", "C5")]
+    out["wall_seconds"] = round(time.perf_counter() - T_START, 1)
     print(json.dumps(out))
-    b.close()
 
 
 if __name__ == "__main__":

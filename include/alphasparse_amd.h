@@ -335,8 +335,8 @@ typedef struct as_search_options {
                                   * shared_memory_op.cc), which the reference keeps out of its white list, are
                                   * searched as well (skeletons G1, G2) */
   int skip_verification;         /* no counterpart in the reference, which times candidates without looking at
-                                  * their result.  0: every candidate runs once on x = 1 and its y is compared with
-                                  * the sums of the rows' values before it is timed; one that differs is logged,
+                                  * their result.  0: every candidate runs once on x[j] = 1 + j % 7 and its y is compared
+                                  * with a host CSR product for that x before it is timed; one that differs is logged,
                                   * counted as failed and cannot win.  1: candidates are only timed */
 } as_search_options;
 /* `input` = the matrix as read (no operator applied); its wave is the wave of every candidate */
