@@ -59,7 +59,7 @@ TEMPLATE_NAMES = ["DIRECT_ATOM_TEMPLATE", "DIRECT_ATOM_TEMPLATE_WARP_COMPRESS", 
 F_INDEX_ARR, F_FIRST_ROW, F_ROW_NUMBER, F_COO_BEGIN, F_COO_BLOCK_SIZE, F_SCALARS = range(6)
 FIELD_NAMES = ["index_arr", "index_of_the_first_row_arr", "row_number_of_block_arr", "coo_begin_index_arr",
                "coo_block_size_arr", "scalars"]
-SLOT_SORTED_ROW_INDEX, SLOT_DENSE_ITEM, SLOT_SHARE_FLAGS, SLOT_COO = 100, 101, 102, 103
+SLOT_SORTED_ROW_INDEX, SLOT_DENSE_ITEM, SLOT_SHARE_FLAGS, SLOT_COO, SLOT_Y_WRITE_INDEX = 100, 101, 102, 103, 104
 V_VAL, V_PADDING_VAL, V_STAGGERED_PADDING_VAL, V_COO_VALUE_CACHE = range(4)
 
 _lib = None
@@ -227,6 +227,9 @@ class MatrixAPI:
             if not info["is_compressed"]:
                 continue
             d[pre + "share_flags"] = self.get_u64(sub, SLOT_SHARE_FLAGS, 0)[0]
+            yw = self.get_u64(sub, SLOT_Y_WRITE_INDEX, 0)
+            if yw is not None:
+                d[pre + "y_write_index"] = (yw[0], DTYPE_NAMES[yw[1]])
             for slot in range(7):
                 sc = self.get_u64(sub, slot, F_SCALARS)
                 if sc is None:

@@ -112,6 +112,10 @@ struct CompressedBlock {
   ValPtr val;                // val_arr            (size == read_index[1]->length)
   ValPtr padding_val;        // padding_val_arr
   ValPtr staggered_val;      // staggered_padding_val_arr
+  // compressed_block_sort (struct.hpp compressed_block_t::is_sorted, y_write_index[0]): the rows inside some BLBs
+  // were re-ordered by length; y_write_index[row after the sort] = row before it, both relative to the sub-matrix
+  bool is_sorted = false;
+  IArr y_write_index;
   // Column slice width when the BLBs were cut at column slice boundaries
   // (COMPRESSED_TBLOCK_LEVEL_COL_DIV_COL_SLICE_PARAM_STRATEGY), else 0.
   uint64_t col_slice = 0;

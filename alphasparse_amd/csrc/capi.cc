@@ -248,6 +248,9 @@ int as_execute_node(as_matrix *m, int node_type, int64_t sub, const long *scalar
     case asx::DENSE_FINE_SORT:
       n.first_row_of_each_sort_band.assign(list, list + n_list);
       break;
+    case asx::COMPRESSED_BLOCK_SORT:
+      n.sort_block_index_arr.assign(list, list + n_list);
+      break;
     case asx::DENSE_FIXED_COL_DIV:
       AS_CHECK(n_scalars >= 1, "need {fixed_col_block_size}");
       n.fixed_col_block_size = scalars[0];
@@ -307,6 +310,10 @@ int64_t as_matrix_get_u64(const as_matrix *m, int64_t sub, int slot, int field, 
   }
   AS_CHECK(it.cb != nullptr, "sub-matrix is not compressed");
   const asx::CompressedBlock &cb = *it.cb;
+  if (slot == AS_SLOT_Y_WRITE_INDEX) {
+    if (!cb.y_write_index.present) return -1;
+    return put_u64(cb.y_write_index.v, cb.y_write_index.dt, out, cap, dtype);
+  }
   if (slot == AS_SLOT_SHARE_FLAGS) {
     std::vector<uint64_t> v{cb.share_row_with_other_block, cb.share_row_with_other_warp, cb.share_row_with_other_thread,
                             cb.read_index.size()};

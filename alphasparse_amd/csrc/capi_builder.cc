@@ -145,6 +145,7 @@ const char *as_template_describe(as_builder *b, int64_t sub) {
   s += "kernal_first_col_index=" + std::to_string(t.kernal_first_col_index) + "\n";
   s += "is_atom_add=" + std::to_string((int)t.is_atom_add) + "\n";
   s += "global_sort_index=" + std::to_string((int)t.global_sort_index) + "\n";
+  s += "local_sort_index=" + std::to_string((int)t.local_sort_index) + "\n";
   for (auto &kv : t.scalar) s += kv.first + "=" + std::to_string(kv.second) + "\n";
   for (auto &a : t.arrays)
     s += "array:" + a.name + "=" + asx::dtype_name(a.a.dt) + "," + std::to_string(a.a.size()) + "," +

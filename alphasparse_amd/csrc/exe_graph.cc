@@ -76,6 +76,13 @@ void execute_exe_node_in_compressed_sub_matrix(Matrix &m, uint64_t sub, const Ex
       AS_CHECK(cb.read_index.size() == 2, "BLB level already exists");
       sep_tblock_level_row_csr(cb, node.row_num_of_each_BLB);
       return;
+    case COMPRESSED_BLOCK_SORT: {  // op_manager API upstream (no node executor there)
+      AS_CHECK(!m.sorted_row_index.present, "a sort inside BLBs excludes a sort of the whole matrix (and remove_empty_rows)");
+      AS_CHECK(cb.read_index.size() == 3, "the BLB level must exist and be the last one");
+      compressed_block_sort(cb, node.sort_block_index_arr.empty() ? iota_ids(cb.read_index[2]->block_num) : node.sort_block_index_arr,
+                            m.items[sub].max_row - m.items[sub].min_row + 1);
+      return;
+    }
     case COMPRESSED_TBLOCK_LEVEL_COL_DIV: {  // exe_graph.cc:1754
       AS_CHECK(cb.read_index.size() == 2, "BLB level already exists");
       if (node.row_group != 0) {  // 2-D tiles (no upstream counterpart)

@@ -29,6 +29,7 @@ struct ExeNode {
   std::vector<std::vector<uint32_t>> nested_block_size;
   std::vector<uint64_t> bin_row_nnz_low_bound;               // DENSE_ROW_COARSE_SORT
   std::vector<uint64_t> first_row_of_each_sort_band;         // DENSE_FINE_SORT (empty: one band)
+  std::vector<uint64_t> sort_block_index_arr;                // COMPRESSED_BLOCK_SORT (empty: every BLB)
   std::vector<uint64_t> row_div_position;                    // DENSE_ROW_DIV
   uint64_t dense_sub_block_id = 0;
   long fixed_col_block_size = 0;                             // DENSE_FIXED_COL_DIV

@@ -302,6 +302,8 @@ std::unique_ptr<CompressedBlock> CompressedBlock::clone() const {
   c->val_dtype = val_dtype;
   c->col_slice = col_slice;
   c->row_group = row_group;
+  c->is_sorted = is_sorted;
+  c->y_write_index = y_write_index;
   // keep aliasing (nnz-div: slots 5/6 alias slot 1, padded values alias val)
   std::vector<std::pair<const Index *, IndexPtr>> seen;
   for (auto &ip : read_index) {

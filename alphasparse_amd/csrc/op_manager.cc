@@ -451,6 +451,63 @@ void sep_tblock_level_row_csr(CompressedBlock &cb, const std::vector<uint32_t> &
   cb.read_index.push_back(p);
 }
 
+// --------------------------------------------------------------------------
+// compressed_block_sort (op_manager.cc:4104-4303): inside each listed BLB the rows are put in order of falling
+// length (index_map_after_sorting, :4499: an insertion sort that only passes strictly shorter rows, i.e. a
+// stable sort) and renumbered first_row, first_row + 1, ...; y_write_index[row after] = row before, both
+// relative to the sub-matrix, typed like the row index array.  Upstream's function leaves
+// compressed_block_t::is_sorted to its caller, and its templates insist on it (e.g. direct_atom_op.cc:156);
+// here the operator sets it.
+// `real_rows`: rows of the sub-matrix before COMPRESSED_ROW_PADDING; a sort that would move one of the rows that
+// padding added in front of a real row is refused (every template cuts its units at the first padding row).
+void compressed_block_sort(CompressedBlock &cb, const std::vector<uint64_t> &sort_block_index_arr, uint64_t real_rows) {
+  AS_CHECK(cb.read_index.size() == 3 && cb.read_index[2]->level == TBLOCK_LEVEL && cb.read_index[2]->ctype == CSR,
+           "the rows inside BLBs are sorted right after the BLB level is made, before any other level");
+  AS_CHECK(cb.row_group == 0 && cb.col_slice == 0, "BLBs that share rows with other BLBs cannot be sorted");
+  AS_CHECK(!cb.is_sorted && !cb.y_write_index.present, "the sub-matrix is already sorted");
+  AS_CHECK(!sort_block_index_arr.empty(), "no BLB to sort");
+  Index &bl = *cb.read_index[2];
+  Index &ri = *cb.read_index[0], &ci = *cb.read_index[1];
+  AS_CHECK(bl.row_number.present && bl.coo_begin.present, "the BLB level has no row counts");
+  AS_CHECK(ri.length == ci.length && sort_block_index_arr.size() <= bl.block_num, "more BLBs listed than there are");
+  const uint64_t rows = bl.max_row - bl.min_row + 1;
+  std::vector<uint64_t> y_write(rows);
+  std::iota(y_write.begin(), y_write.end(), 0);
+  std::vector<bool> done(bl.block_num, false);
+  std::vector<uint64_t> &row = ri.index_arr.v, &col = ci.index_arr.v;
+  ValVec &val = *cb.val;
+  for (uint64_t b : sort_block_index_arr) {
+    AS_CHECK(b < bl.block_num && !done[b], "BLB number out of range or listed twice");
+    done[b] = true;
+    const uint64_t k0 = bl.coo_begin[b], k1 = bl.coo_begin[b + 1], first = bl.first_row[b], n = bl.row_number[b];
+    AS_CHECK(k1 > k0 && first + n <= rows, "malformed BLB");
+    std::vector<uint64_t> len(n, 0), off(n + 1, 0);
+    for (uint64_t k = k0; k < k1; k++) {
+      AS_CHECK(row[k] >= first && row[k] < first + n, "element outside the rows of its BLB");
+      len[row[k] - first]++;
+    }
+    for (uint64_t r = 0; r < n; r++) off[r + 1] = off[r] + len[r];
+    std::vector<uint64_t> order(n);  // new local row -> old local row
+    std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(), [&](uint64_t x, uint64_t y) { return len[x] > len[y]; });
+    std::vector<uint64_t> ncol(col.begin() + k0, col.begin() + k1);
+    ValVec nval(val.begin() + k0, val.begin() + k1);
+    uint64_t pos = k0;
+    for (uint64_t nr = 0; nr < n; nr++) {
+      for (uint64_t k = off[order[nr]]; k < off[order[nr] + 1]; k++, pos++) {
+        row[pos] = first + nr;
+        col[pos] = ncol[k];
+        val[pos] = nval[k];
+      }
+      y_write[first + nr] = first + order[nr];
+      AS_CHECK((first + nr >= real_rows) == (first + order[nr] >= real_rows),
+               "the sort would mix rows added by row padding with rows of the matrix (padding_row_length above a row's length)");
+    }
+  }
+  cb.y_write_index.assign(std::move(y_write), ri.index_arr.dt);
+  cb.is_sorted = true;
+}
+
 void default_sep_tblock_level_row_csr(CompressedBlock &cb) {
   AS_CHECK(cb.read_index.size() == 2, "BLB level already exists");
   sep_tblock_level_row_csr(cb, {(uint32_t)sub_rows(cb)});

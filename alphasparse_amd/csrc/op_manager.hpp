@@ -22,6 +22,9 @@ std::vector<std::unique_ptr<Matrix>> long_short_row_decomposition(const Matrix &
 // total_dense_block_sort (op_manager.cc:4780; banded form :4871): rows by length, longest first, rows of equal
 // length in their previous order (upstream sorts by insertion); with bands, inside every band of rows
 // [first[i], first[i+1]) (the last band ends with the matrix).  sorted_row_index[new] = old.
+// op_manager.cc:4104 compressed_block_sort: rows of the listed BLBs by falling length, permutation in y_write_index
+void compressed_block_sort(CompressedBlock &cb, const std::vector<uint64_t> &sort_block_index_arr,
+                           uint64_t real_rows = ~0ull);
 void total_dense_block_sort(Matrix &m, const std::vector<uint64_t> &first_row_of_each_sort_band = {});
 // global_padding_position (op_manager.hpp:13): where total_row_level_padding* puts the rows it adds
 enum PaddingPosition { TOP_PADDING = 0, END_PADDING = 1 };

@@ -53,6 +53,9 @@ struct Template {
   uint64_t kernal_first_row_index = 0, kernal_first_col_index = 0;
   bool is_atom_add = false;
   bool global_sort_index = false;
+  // the rows inside BLBs were sorted (compressed_block_sort): row numbers go through y_write_index, which is
+  // relative to the sub-matrix (upstream local_sort_index, e.g. direct_atom_op.cc:153-175)
+  bool local_sort_index = false;
   // template specific scalars (effective_TLB_num, thread_block_size_in_block, ...)
   std::map<std::string, uint64_t> scalar;
   std::vector<TArr> arrays;       // metadata arrays, in kernel-argument order

@@ -59,6 +59,15 @@ uint64_t effective_unit_num(const Matrix &m, uint64_t sub, const std::vector<uin
 }
 
 bool apply_global_sort(const Matrix &m, uint64_t sub, std::vector<uint64_t> &unit_row, uint64_t effective) {
+  const CompressedBlock &cb = *m.items[sub].cb;
+  if (cb.y_write_index.present) {
+    // rows sorted inside BLBs: back to the rows of the sub-matrix; they stay relative to its first row, and a
+    // sort of the whole matrix (or the map of remove_empty_rows) may follow below
+    for (uint64_t u = 0; u < effective; u++) {
+      AS_CHECK(unit_row[u] < cb.y_write_index.size(), "row outside the permutation of the BLB sort");
+      unit_row[u] = cb.y_write_index[unit_row[u]];
+    }
+  }
   if (!m.sorted_row_index.present) return false;
   uint64_t first = m.items[sub].min_row;
   for (uint64_t u = 0; u < effective; u++) {
@@ -80,6 +89,7 @@ void init_template_common(Template &t, TemplateType type, const Matrix &m, uint6
   t.kernal_first_row_index = m.items[sub].min_row;
   t.kernal_first_col_index = m.items[sub].min_col;
   t.origin_nnz = m.items[sub].end_coo - m.items[sub].begin_coo + 1;
+  t.local_sort_index = m.items[sub].cb->y_write_index.present;
   const CompressedBlock &cb = *m.items[sub].cb;
   t.padding_arr_size = cb.padding_val ? cb.padding_val->size() : (cb.val ? cb.val->size() : 0);
 }

@@ -201,6 +201,8 @@ std::unique_ptr<Template> init(const Matrix &m, uint64_t sub) {
   if (m.sorted_row_index.present) {
     t->global_sort_index = true;
     add("row_index_before_sort", m.sorted_row_index.v, m.sorted_row_index.dt);
+  } else if (cb.y_write_index.present) {  // rows sorted inside BLBs: the permutation is relative to the sub-matrix
+    add("row_index_before_sort", cb.y_write_index.v, cb.y_write_index.dt);
   }
   t->val_arr = *cb.staggered_val;
   t->col_index_arr = cb.read_index[6]->index_arr;
@@ -261,7 +263,10 @@ std::string kernel_source(const Template &t) {
   s += "      sum = as_group_sum<" + Rs + ">(sum);\n";
   s += "      if ((threadIdx.x % " + Rs + "u) == " + Rs + "u - 1u && row < " + std::to_string(t.sc("effective_row_num")) +
        "u && res_end > res_begin)\n      {\n";
-  s += "        unsigned int global_row_index = row + " + std::to_string(t.kernal_first_row_index) + "u;\n";
+  if (t.local_sort_index && !t.global_sort_index)
+    s += "        unsigned int global_row_index = row_index_before_sort[row] + " + std::to_string(t.kernal_first_row_index) + "u;\n";
+  else
+    s += "        unsigned int global_row_index = row + " + std::to_string(t.kernal_first_row_index) + "u;\n";
   if (t.global_sort_index) s += "        global_row_index = row_index_before_sort[global_row_index];\n";
   s += t.is_atom_add ? "        as_atomic_add(device_y_arr + global_row_index, sum);\n"
                      : "        as_stnt(device_y_arr + global_row_index, sum);\n";

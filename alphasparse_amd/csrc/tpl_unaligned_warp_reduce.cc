@@ -145,6 +145,8 @@ std::unique_ptr<Template> make(TemplateType type, const Matrix &m, uint64_t sub)
   if (m.sorted_row_index.present) {
     t->global_sort_index = true;
     add("row_index_before_sort", m.sorted_row_index.v, m.sorted_row_index.dt, true);
+  } else if (cb.y_write_index.present) {  // rows sorted inside BLBs: the permutation is relative to the sub-matrix
+    add("row_index_before_sort", cb.y_write_index.v, cb.y_write_index.dt, true);
   }
   // interleave: element k of TLB lane -> wlb * W * s + lane + k * W   (:282-291)
   t->col_index_arr.assign(std::vector<uint64_t>(u.col.size()), cb.read_index[1]->index_arr.dt);
@@ -176,6 +178,8 @@ std::string source(const Template &t, bool grid_stride) {
   const std::string mt = word == 64 ? "as_u64" : "as_u32";
   std::string write_row = t.global_sort_index
                               ? "row_index_before_sort[" + std::to_string(t.kernal_first_row_index) + "u + (ROW)]"
+                          : t.local_sort_index
+                              ? "(" + std::to_string(t.kernal_first_row_index) + "u + row_index_before_sort[(ROW)])"
                               : "(" + std::to_string(t.kernal_first_row_index) + "u + (ROW))";
   std::string S;
   S += "extern \"C\" __global__ void __launch_bounds__(" + B + ") spmv_" + id + "(" + kernel_signature(t) + ")\n{\n";

@@ -54,10 +54,17 @@ def skeleton(name, **kw):
     raise ValueError("unknown skeleton " + name)
 
 
-def apply_skeleton(matrix, sub, name, **kw):
-    """Run the skeleton's strategies on one compressed sub-matrix and complete the blocking."""
+BLB_LEVEL_STRATEGIES = (K.COMPRESSED_TBLOCK_LEVEL_ROW_DIV_EVENLY, K.COMPRESSED_TBLOCK_LEVEL_ROW_DIV_ACC_TO_LEAST_NNZ)
+
+
+def apply_skeleton(matrix, sub, name, block_sort=None, **kw):
+    """Run the skeleton's strategies on one compressed sub-matrix and complete the blocking.
+    block_sort: None, or the list of BLBs whose rows are sorted by falling length right after the BLB level is
+    made (COMPRESSED_BLOCK_SORT; an empty list = every BLB)."""
     strategies, templates = skeleton(name, **kw)
     for s, p in strategies:
         matrix.execute_strategy(s, sub, p)
+        if block_sort is not None and s in BLB_LEVEL_STRATEGIES:
+            matrix.execute_node(K.COMPRESSED_BLOCK_SORT, sub, lst=block_sort)
     matrix.complete_blocking(sub)
     return templates

@@ -86,7 +86,9 @@ enum as_special_slot {
   AS_SLOT_SORTED_ROW_INDEX = 100, /* sparse_struct_t::sorted_row_index (sub ignored) */
   AS_SLOT_DENSE_ITEM = 101,       /* {min_row,max_row,min_col,max_col,begin_coo,end_coo,is_col_blocked} */
   AS_SLOT_SHARE_FLAGS = 102,      /* {share_row_with_other_block, _warp, _thread, read_index.size()} */
-  AS_SLOT_COO = 103               /* field 0/1 = coo_row_index_cache / coo_col_index_cache (sub ignored) */
+  AS_SLOT_COO = 103,              /* field 0/1 = coo_row_index_cache / coo_col_index_cache (sub ignored) */
+  AS_SLOT_Y_WRITE_INDEX = 104     /* compressed_block_t::y_write_index[0] (struct.hpp): the permutation of
+                                   * compressed_block_sort, absent (-1) without it */
 };
 enum as_value_array { AS_V_VAL, AS_V_PADDING_VAL, AS_V_STAGGERED_PADDING_VAL, AS_V_COO_VALUE_CACHE };
 
@@ -174,6 +176,10 @@ int as_matrix_write_binary_file(const as_matrix *m, const char *path);
  *   COMPRESSED_TBLOCK_LEVEL_ROW_DIV list = row count of every BLB
  *   COMPRESSED_TBLOCK_LEVEL_COL_DIV / WARP_LEVEL_ROW_DIV / WARP_LEVEL_COL_DIV
  *                                   counts[i] = number of entries of parent i, list = all entries, concatenated
+ *   COMPRESSED_BLOCK_SORT           list = sort_block_index_arr: the BLBs whose rows are sorted by falling length
+ *                                   (op_manager.cc:4104 compressed_block_sort; the reference has the operator and its
+ *                                   templates read the permutation, but no node executor); right after the BLB
+ *                                   level is made; an empty list = every BLB
  *   DENSE_ROW_COARSE_SORT           list = bin_row_nnz_low_bound
  *   DENSE_ROW_DIV                   list = row_div_position
  *   COMPRESS, COMPRESSED_THREAD_LEVEL_ROW_DIV   no parameters                                       */

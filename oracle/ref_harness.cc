@@ -165,6 +165,17 @@ int ref_execute_node(void *hv, int node_type, int64_t sub, const long *scalars, 
     case COMPRESS:
       compress_dense_view(h->m);
       return 0;
+    case COMPRESSED_BLOCK_SORT: {
+      // upstream has the operator (op_manager.cc:4104) but no node executor for it; its templates insist on
+      // compressed_block_t::is_sorted (e.g. direct_atom_op.cc:156), which the operator leaves to its caller
+      compressed_block_t *cb = h->m->block_coor_table.item_arr[sub]->compressed_block_ptr;
+      vector<unsigned long> blocks(list, list + n_list);
+      if (blocks.empty())
+        for (unsigned long b = 0; b < cb->read_index[2]->block_num; b++) blocks.push_back(b);
+      compressed_block_sort(cb, blocks);
+      cb->is_sorted = true;
+      return 0;
+    }
     case COMPRESSED_ROW_PADDING: {
       exe_compress_row_padding_param_t p;
       p.multiply = scalars[0];
@@ -364,6 +375,10 @@ int64_t ref_get_u64(void *hv, int64_t sub, int slot, int field, uint64_t *out, u
   }
   compressed_block_t *cb = it->compressed_block_ptr;
   if (cb == NULL) return -2;
+  if (slot == 104) {  // y_write_index[0] of compressed_block_sort
+    if (cb->y_write_index.empty()) return -1;
+    return put(cb->y_write_index[0]->index_arr, cb->y_write_index[0]->index_data_type, cb->y_write_index[0]->length, out, cap, dtype);
+  }
   if (slot == 102) {
     uint64_t v[4] = {cb->share_row_with_other_block, cb->share_row_with_other_warp, cb->share_row_with_other_thread,
                      cb->read_index.size()};
@@ -434,6 +449,7 @@ struct TplView {
   v.scalars.push_back({"kernal_first_row_index", (T)->kernal_first_row_index});                     \
   v.scalars.push_back({"kernal_first_col_index", (T)->kernal_first_col_index});                     \
   v.scalars.push_back({"global_sort_index", (uint64_t)(T)->global_sort_index});                     \
+  v.scalars.push_back({"local_sort_index", (uint64_t)(T)->local_sort_index});                       \
   ARRN(T, col_index_arr);                                                                           \
   v.val = (T)->val_arr; v.val_dt = (T)->data_type_of_val_arr; v.val_n = (T)->size_of_val_arr;
 

@@ -80,6 +80,15 @@ FORMAT_CASES = [
     ("finesort_irr_ell", "irr", FINE_SORT, "S5", {"wave": 32}),
     ("bandsort_pl_csr5", "pl", BAND_SORT, "S9", {"t": 3}),
     ("bandsort_irr_longrow", "irr", BAND_SORT, "S8", {"b": 32}),
+    # compressed_block_sort (op_manager.cc:4104): the rows inside all or some BLBs by falling length, right after the
+    # BLB level is made; the permutation (y_write_index) goes through every template's row numbers
+    ("blocksort_pl_sell32", "pl", [], "S1", {"m": 32, "block_sort": []}),
+    ("blocksort_pl_s2", "pl", [], "S2", {"m": 32, "len": 1, "s": 3, "block_sort": [0, 2, 4]}),
+    ("blocksort_pl_s3", "pl", [], "S3", {"n": 128, "s": 3, "block_sort": []}),
+    ("blocksort_pl_s6", "pl", [], "S6", {"m": 4, "len": 1, "c": 8, "block_sort": []}),
+    ("blocksort_pl_long_s7", "pl_long", [], "S7", {"n": 700, "c": 64, "block_sort": []}),
+    ("blocksort_pl_base_direct", "pl", [], "B1", {"m": 40, "w": 8, "block_sort": []}),
+    ("blocksort_pl_base_lds", "pl", [], "B2", {"n": 200, "w": 4, "s": 3, "block_sort": [1]}),
     # configuration 1 (4096 x 4096, 8 per row) through the ELL graph and through the SELL graph the search returns for it
     ("c1_ell", "c1", [], "S5", {"wave": 32}),
     ("c1_sell512", "c1", [], "S1", {"m": 512}),

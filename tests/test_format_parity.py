@@ -116,7 +116,7 @@ RANDOM_SEQS = {
 REFERENCE_DONE = "reference side finished"
 
 
-def live_compare(skel, seed, sort):
+def live_compare(skel, seed, sort, block_sort=None):
     """Product vs upstream on one random matrix; returns the list of differences.  The upstream side runs first
     and to its end (operators, template initialisation, every dump) and its end is announced on stderr: whatever
     ends the process after that line is the product's doing."""
@@ -130,7 +130,7 @@ def live_compare(skel, seed, sort):
         if sort:
             m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
         m.execute_strategy(K.COMPRESS_NONE)
-        return SK.apply_skeleton(m, 0, skel, **RANDOM_SEQS[skel])
+        return SK.apply_skeleton(m, 0, skel, block_sort=block_sort, **RANDOM_SEQS[skel])
 
     ref = ref_lib.RefMatrix(rows, cols, r, c, v, K.FLOAT)
     templates = build(ref)
@@ -175,6 +175,53 @@ def test_format_matches_upstream_live(skel, seed, sort):
     if rejected:
         pytest.skip("upstream rejects this operator sequence: " + rejected[:300])
     assert p.returncode == 0, "return code %d\n" % p.returncode + p.stdout[-3000:] + p.stderr[-2000:]
+
+
+@pytest.mark.parametrize("skel", ["S1", "S2", "S3", "S6", "S7", "B1", "B2"])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_block_sort_matches_upstream_live(skel, seed):
+    """compressed_block_sort on random matrices, on every BLB (even seeds) or on BLBs 0 and 1, through the skeletons
+    that make the BLB level themselves; the format arrays, y_write_index and every template array against upstream."""
+    _live()
+    import subprocess
+    import sys
+    code = ("import sys; sys.path[:0] = %r; import test_format_parity as t; d = t.live_compare(%r, %d, False, %r); "
+            "print('\\n'.join(d)); sys.exit(1 if d else 0)") % (sys.path[:4], skel, seed, [] if seed % 2 == 0 else [0, 1])
+    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    rejected = upstream_rejected(p.stderr) if p.returncode != 0 else None
+    if rejected:
+        pytest.skip("upstream rejects this operator sequence: " + rejected[:300])
+    assert p.returncode == 0, "return code %d\n" % p.returncode + p.stdout[-3000:] + p.stderr[-2000:]
+
+
+def test_block_sort_known_answer():
+    """What the operator must do, stated without the upstream code: BLBs of 4 rows, rows of BLB 1 by falling length
+    (ties keep their order), renumbered; y_write_index[row after] = row before."""
+    lens = [2, 1, 3, 1, 1, 4, 4, 2]
+    rows, cols, r, c, v, _ = cases._steps(lens, 16, 3)
+    m = product_matrix(rows, cols, r, c, v.astype(np.float64), K.DOUBLE)
+    m.execute_strategy(K.COMPRESS_NONE)
+    m.execute_strategy(K.COMPRESSED_TBLOCK_LEVEL_ROW_DIV_EVENLY, 0, (4,))
+    before_col = m.get_u64(0, 1, 0)[0].copy()
+    m.execute_node(K.COMPRESSED_BLOCK_SORT, 0, lst=[1])
+    assert m.get_u64(0, K.SLOT_Y_WRITE_INDEX, 0)[0].tolist() == [0, 1, 2, 3, 5, 6, 7, 4]
+    row = m.get_u64(0, 0, 0)[0].astype(np.int64)
+    assert np.bincount(row).tolist() == [2, 1, 3, 1, 4, 4, 2, 1]
+    off = np.concatenate([[0], np.cumsum(lens)])
+    want_col = np.concatenate([before_col[:off[4]]] + [before_col[off[o]:off[o + 1]] for o in (5, 6, 7, 4)])
+    assert np.array_equal(m.get_u64(0, 1, 0)[0], want_col)
+    with pytest.raises(A.AlphaSparseError):
+        m.execute_node(K.COMPRESSED_BLOCK_SORT, 0, lst=[0])              # sorted already
+    m2 = product_matrix(rows, cols, r, c, v.astype(np.float64), K.DOUBLE)
+    m2.execute_strategy(K.COMPRESS_NONE)
+    with pytest.raises(A.AlphaSparseError):
+        m2.execute_node(K.COMPRESSED_BLOCK_SORT, 0, lst=[0])             # no BLB level yet
+    m3 = product_matrix(rows, cols, r, c, v.astype(np.float64), K.DOUBLE)
+    m3.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+    m3.execute_strategy(K.COMPRESS_NONE)
+    m3.execute_strategy(K.COMPRESSED_TBLOCK_LEVEL_ROW_DIV_EVENLY, 0, (4,))
+    with pytest.raises(A.AlphaSparseError):
+        m3.execute_node(K.COMPRESSED_BLOCK_SORT, 0, lst=[0])             # excludes a sort of the whole matrix
 
 
 def test_live_skip_rule_does_not_hide_a_crash_of_the_product():

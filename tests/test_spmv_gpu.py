@@ -149,6 +149,13 @@ GPU_CASES = [
     # total_dense_block_sort over all rows and inside bands of rows: y goes back through the permutation
     ("pl", FINE_SORT(), "S1", {"m": 64}, ({},)), ("pl", FINE_SORT(0, 1000, 1001, 2500), "S5", {}, ({},)),
     ("irr", FINE_SORT(0, 17), "T1", {"slice": 1024, "group": 512, "b": 300}, ({},)), ("pl", FINE_SORT(0, 700), "T2", {"slice": 512, "group": 16, "b": 1024}, ({},)),
+    # compressed_block_sort: rows inside the BLBs by falling length, y through y_write_index (direct stores, LDS
+    # row sums and atomics alike); all BLBs or a few of them
+    ("pl", [], "S1", {"m": 128, "block_sort": []}, VEC), ("irr", [], "S1", {"m": 64, "block_sort": [0, 3, 7]}, ({},)),
+    ("pl", [], "S2", {"m": 64, "len": 1, "s": 4, "block_sort": []}, RED), ("pl", [], "S3", {"n": 512, "s": 3, "block_sort": []}, ({},)),
+    ("pl", [], "S6", {"m": 4, "len": 1, "c": 16, "block_sort": []}, ({},)), ("pl", [], "S7", {"n": 896, "c": 64, "block_sort": [1, 2]}, ({},)),
+    ("pl", [], "B1", {"m": 96, "w": 8, "block_sort": []}, ({},)), ("pl", [], "B2", {"n": 512, "w": 8, "s": 3, "block_sort": []}, ({},)),
+    ("uni40", COLDIV(700), "S1", {"m": 64, "block_sort": []}, ({},)), ("pl", D3[1:], "S1", {"m": 64, "block_sort": []}, ({},)),
     # the two general templates (outside the white list)
     ("uni40", [], "B1", {"m": 64, "w": 16}, ({}, {"thread_num_in_block": 64}, {"thread_num_in_block": 1024})),
     ("pl", SORT, "B1", {"m": 96, "w": 8}, ({},)), ("pl", D3, "B1", {"m": 64, "w": 8}, ({},)), ("fem", [], "B1", {"m": 30, "w": 6}, ({},)),
@@ -183,7 +190,7 @@ GPU_CASES = [
 
 @pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
 @pytest.mark.parametrize("mat,dense,skel,kw,launches", GPU_CASES,
-                         ids=["%s-%s%s-%s" % (c[0], "D" if c[1] else "", c[2], "_".join("%s%s" % kv for kv in c[3].items())) for c in GPU_CASES])
+                         ids=["%s-%s%s-%s" % (c[0], "D" if c[1] else "", c[2], "_".join("%s%s" % (k, "".join(map(str, v)) if isinstance(v, list) else v) for k, v in c[3].items())) for c in GPU_CASES])
 def test_spmv_matches_cpu_csr(gpu, mat, dense, skel, kw, launches, vdt):
     run_case(gpu, MATS[mat](), vdt, dense, skel, kw, launches)
 
