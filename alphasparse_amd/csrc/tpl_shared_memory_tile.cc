@@ -41,6 +41,7 @@ static const uint64_t kLaneElems = 8;       // consecutive elements of one lane 
 static const uint64_t kRunUnit = 64 * kLaneElems;  // elements of one wavefront step
 static const unsigned kNewPieceBit = 14;    // lane word: bit 14 + j = element j (1..7) starts a new piece
 static const unsigned kStoreBit = 14 + kLaneElems;  // bit 22 + j = a sum emitted at element j (0..7) is the piece's only one
+static const unsigned kBetweenRunsBatch = 8; // requests a lane keeps in flight in the write-back and in the slice copy
 static const unsigned kBatch = 1;           // wavefront steps whose loads are in flight together (a step is 8
                                             // elements per lane, 4-6 loads: deeper batches measured slower)
 
@@ -360,26 +361,56 @@ std::string kernel_source(const Template &t) {
   s += "        " + code_of_meta_read(t, "run_piece_begin", "piece_end", "next_run");
   s += "      }\n";
   s += "      __syncthreads();\n";  // every wavefront is done with the previous run
+  // Between two runs a workgroup writes the finished run back (a table read and one atomic per piece) and, when the
+  // slice changes, copies the new slice of x into LDS.  Written as plain loops, both are chains of memory round
+  // trips: the compiler waits for an atomic to complete before it lets anything overwrite the atomic's data
+  // registers, and for each load of the copy before its LDS store, so every iteration costs a trip (or two) to
+  // memory.  Here a lane first requests everything it needs -- the sums, the places and the addresses of its
+  // pieces -- then issues its atomics back to back from registers nobody writes in between; the slice copy
+  // requests a batch of loads before it stores the first.
+  const uint64_t wb_batch = std::min<uint64_t>(kBetweenRunsBatch, std::max<uint64_t>(1, (R + t.thread_num_in_block - 1) / t.thread_num_in_block));
+  const std::string Ws = std::to_string(wb_batch);
   // write-back of the run that ended: consecutive lanes take consecutive pieces (rows in rising order)
-  s += "      for (unsigned int i = threadIdx.x; i < done_end - done_begin; i += " + B + ")\n      {\n";
-  s += "        const " + vt + " sum = piece_sum[i];\n";
-  s += "        piece_sum[i] = 0;\n";
-  s += "        if (sum != 0)\n        {\n";
-  s += "          unsigned int at = done_begin + i, place;\n";
-  s += "          " + code_of_meta_read(t, "piece_target", "place", "at");
-  s += "          as_atomic_add(" + target + " + place, sum);\n";
-  s += "        }\n      }\n";
+  s += "      for (unsigned int i0 = threadIdx.x; i0 < done_end - done_begin; i0 += " + B + " * " + Ws + "u)\n      {\n";
+  s += "        typedef __attribute__((address_space(1))) " + vt + " *global_ptr_t;\n";
+  s += "        " + vt + " sum[" + Ws + "];\n        unsigned int place[" + Ws + "];\n        global_ptr_t where[" + Ws + "];\n";
+  s += "        #pragma unroll\n        for (int j = 0; j < " + Ws + "; j++)\n        {\n";
+  s += "          const unsigned int i = i0 + j * " + B + ";\n";
+  s += "          sum[j] = 0;\n          place[j] = 0u;\n";
+  s += "          if (i < done_end - done_begin)\n          {\n";
+  s += "            sum[j] = piece_sum[i];\n            piece_sum[i] = 0;\n";
+  s += "            const unsigned int at = done_begin + i;\n";
+  s += "            " + code_of_meta_read(t, "piece_target", "place[j]", "at");
+  s += "          }\n        }\n";
+  // (the empty asm pins every address in registers of its own here, ahead of the atomics)
+  s += "        #pragma unroll\n        for (int j = 0; j < " + Ws + "; j++)\n        {\n          where[j] = (global_ptr_t)(" + target + " + place[j]);\n          asm volatile(\"\" : \"+v\"(where[j]));\n        }\n";
+  s += "        __builtin_amdgcn_sched_barrier(0);\n";  // every address is in its registers before the first atomic goes out
+  s += "        #pragma unroll\n        for (int j = 0; j < " + Ws + "; j++)\n";
+  s += "          if (sum[j] != 0) __builtin_amdgcn_global_atomic_fadd_" + std::string(t.val_dtype == DOUBLE ? "f64" : "f32") + "(where[j], sum[j]);\n";
+  s += "      }\n";
   s += "      done_begin = piece_begin; done_end = piece_end;\n";
   s += "      if (run < run_end && slice != cur_slice)\n      {\n";
   s += "        const unsigned int col0 = slice * " + Ss + ";\n";
   s += "        const unsigned int slice_len = min(" + Ss + ", " + std::to_string(x_len) + "u - col0);\n";
+  const std::string Ks2 = std::to_string(kBetweenRunsBatch);
   if (wide_copy) {
     // 16 bytes per lane and load: the 64 lanes of a load read one contiguous kilobyte
-    s += "        for (unsigned int i = threadIdx.x * " + Cs + "u; i + " + Cs + "u <= slice_len; i += " + B + " * " + Cs + "u)\n";
-    s += "          *(val16_t *)(x_slice + i) = *(const val16_t *)(x_sub + col0 + i);\n";
+    s += "        for (unsigned int i0 = threadIdx.x * " + Cs + "u; i0 + " + Cs + "u <= slice_len; i0 += " + Ks2 + "u * " + B + " * " + Cs + "u)\n        {\n";
+    s += "          val16_t part[" + Ks2 + "];\n";
+    s += "          #pragma unroll\n          for (int j = 0; j < " + Ks2 + "; j++)\n";
+    s += "            if (i0 + j * " + B + " * " + Cs + "u + " + Cs + "u <= slice_len) part[j] = *(const val16_t *)(x_sub + col0 + i0 + j * " + B + " * " + Cs + "u);\n";
+    s += "          #pragma unroll\n          for (int j = 0; j < " + Ks2 + "; j++)\n";
+    s += "            if (i0 + j * " + B + " * " + Cs + "u + " + Cs + "u <= slice_len) *(val16_t *)(x_slice + i0 + j * " + B + " * " + Cs + "u) = part[j];\n";
+    s += "        }\n";
     s += "        if (threadIdx.x < slice_len % " + Cs + "u) x_slice[slice_len / " + Cs + "u * " + Cs + "u + threadIdx.x] = x_sub[col0 + slice_len / " + Cs + "u * " + Cs + "u + threadIdx.x];\n";
   } else {
-    s += "        for (unsigned int i = threadIdx.x; i < slice_len; i += " + B + ") x_slice[i] = x_sub[col0 + i];\n";
+    s += "        for (unsigned int i0 = threadIdx.x; i0 < slice_len; i0 += " + Ks2 + "u * " + B + ")\n        {\n";
+    s += "          " + vt + " one[" + Ks2 + "];\n";
+    s += "          #pragma unroll\n          for (int j = 0; j < " + Ks2 + "; j++)\n";
+    s += "            if (i0 + j * " + B + " < slice_len) one[j] = x_sub[col0 + i0 + j * " + B + "];\n";
+    s += "          #pragma unroll\n          for (int j = 0; j < " + Ks2 + "; j++)\n";
+    s += "            if (i0 + j * " + B + " < slice_len) x_slice[i0 + j * " + B + "] = one[j];\n";
+    s += "        }\n";
   }
   s += "        cur_slice = slice;\n      }\n";
   s += "      __syncthreads();\n";

@@ -103,10 +103,13 @@ def build_pinned(m, pin):
         b.set_launch(0, thread_num_in_block=int(threads), vec_width=int(vec))
         return b, res
     dense, *strips = pin.split("|")
+    serial = True
     for op in filter(None, dense.split("+")):
         if op == "sort":
             m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
             res.dense_strategy = 3
+        elif op == "par":
+            serial = False        # the strip kernels on concurrent streams instead of one after the other
         elif op.startswith("div"):
             low = int(op[3:])
             m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (low, low, 2, 0))
@@ -131,7 +134,7 @@ def build_pinned(m, pin):
             raise SystemExit("bench.py: the column-run form does not apply to strip %d" % s)
         if launch:
             b.set_launch(s, thread_num_in_block=launch[0], vec_width=launch[1] if len(launch) > 1 else 0)
-    b.set_serial_launch(True)
+    b.set_serial_launch(serial)
     return b, res
 
 
@@ -296,7 +299,7 @@ def main():
                          "winners and a configuration is skipped when the budget would be exceeded")
     ap.add_argument("--pin", default=None, metavar="SKELETON,THREADS,VEC | DENSE|STRIP0|STRIP1...",
                     help="with --workload: skip the search and run a fixed graph: S5,128,1 (ELL, 128 threads, 1 row per lane; S5,128,1,rel with 16-bit relative columns), or with "
-                         "row strips 'sort+div16|T1@1024|S1:m=128@128' = coarse sort, two strips at row length 16, strip 0 "
+                         "row strips 'sort+div16|T1@1024|S1:m=128@128' = coarse sort, two strips at row length 16 ('+par': strip kernels on concurrent streams), strip 0 "
                          "skeleton T1 with 1024 threads, strip 1 skeleton S1 (m = 128) with 128 threads, kernels one after "
                          "the other ('@1024,runs': the tile template in its column-run form); used for profiling runs that must all "
                          "measure the same kernels")
