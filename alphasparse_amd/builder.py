@@ -36,6 +36,7 @@ def _bind(L):
     L.as_builder_set_relative_columns.argtypes = [vp, C.c_int64]
     L.as_builder_set_diagonal_columns.argtypes = [vp, C.c_int64]
     L.as_builder_set_column_runs.argtypes = [vp, C.c_int64]
+    L.as_builder_set_row_ownership.argtypes = [vp, C.c_int64]
     L.as_builder_set_x.argtypes = [vp, vp]
     L.as_builder_set_serial_launch.argtypes = [vp, C.c_int]
     L.as_builder_time_sub_matrix.argtypes = [vp, C.c_int64, C.c_uint64, C.POINTER(C.c_float), C.POINTER(C.c_uint64),
@@ -124,6 +125,12 @@ class Builder:
         eight elements + a byte of run starts); True when applied (upload again), False when the template is another
         one or the element stream would not get shorter."""
         return bool(self._chk(self._L.as_builder_set_column_runs(self._h, sub)))
+
+    def set_row_ownership(self, sub):
+        """Tile template under row ownership (every row group belongs to one workgroup, rows stored to y without
+        atomics); True when applied (upload again), False when the template is another one or the form does not
+        fit the sub-matrix."""
+        return bool(self._chk(self._L.as_builder_set_row_ownership(self._h, sub)))
 
     def get_launch(self, sub):
         out = (C.c_long * 4)()

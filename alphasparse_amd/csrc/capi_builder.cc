@@ -94,6 +94,13 @@ int as_builder_set_diagonal_columns(as_builder *b, int64_t sub) {
   AS_API_END(-1)
 }
 
+int as_builder_set_row_ownership(as_builder *b, int64_t sub) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b && sub >= 0, "bad argument");
+  return asx::set_row_ownership(*b->b, (uint64_t)sub) ? 1 : 0;
+  AS_API_END(-1)
+}
+
 int as_builder_set_column_runs(as_builder *b, int64_t sub) {
   AS_API_BEGIN
   AS_CHECK(b && b->b && sub >= 0, "bad argument");

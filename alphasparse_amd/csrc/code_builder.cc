@@ -131,11 +131,34 @@ bool set_diagonal_columns(Builder &b, uint64_t sub) {
   return true;
 }
 
+bool set_row_ownership(Builder &b, uint64_t sub) {
+  AS_CHECK(b.matrix != nullptr && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template");
+  Template &old = *b.subs[sub].tpl;
+  if (old.type != SHARED_MEMORY_TILE_TEMPLATE || old.own_rows) return false;
+  std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, old.col_runs, true);
+  if (!t) return false;
+  // the zero-valued elements that close lanes where a row of a group is missing from a slice must stay few
+  if ((double)t->val_arr.size() > 1.05 * (double)old.val_arr.size()) return false;
+  try_all_compress(*t);
+  t->y_needs_clear = template_needs_cleared_y(*t, *b.matrix, sub);
+  t->thread_num_in_block = old.thread_num_in_block;
+  set_default_launch(*t);
+  if (b.subs[sub].uploaded) {
+    as_hip_device_sync();
+    free_sub_arrays(b.subs[sub]);
+    b.subs[sub].uploaded = false;
+  }
+  b.subs[sub].tpl = std::move(t);
+  invalidate(b);
+  return true;
+}
+
 bool set_column_runs(Builder &b, uint64_t sub) {
   AS_CHECK(b.matrix != nullptr && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template");
   Template &old = *b.subs[sub].tpl;
   if (old.type != SHARED_MEMORY_TILE_TEMPLATE || old.col_runs) return false;
-  std::unique_ptr<Template> t = init_tile_template_with_column_runs(*b.matrix, sub);
+  std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, true, old.own_rows);
+  if (!t) return false;
   // worth it when the element stream gets shorter: the padding that closes lanes must not eat the 7 bytes per
   // lane that the columns save
   const double vs = (double)dtype_size(old.val_dtype);

@@ -61,6 +61,10 @@ bool set_diagonal_columns(Builder &b, uint64_t sub);
 // keeps it when the element stream gets shorter by at least 2 %; false (template unchanged) otherwise, or when
 // the sub-matrix has another template.  The launch setting is kept.
 bool set_column_runs(Builder &b, uint64_t sub);
+// Rebuilds the tile template of a sub-matrix under row ownership (init_tile_template_variant; the column-run form
+// is kept when it is in place); false (template unchanged) when the sub-matrix has another template, the form
+// is in place already or it does not fit the sub-matrix.  The launch setting is kept.
+bool set_row_ownership(Builder &b, uint64_t sub);
 // Whole module: preamble + every spmv_<sub> (code_of_kernal_define, build_main_file's kernel part)
 std::string build_module_source(const Builder &b);
 void compile_builder(Builder &b);                 // hipRTC, no GPU needed (compile_spmv_code, executor.cc:61)

@@ -103,6 +103,7 @@ std::string convert_template_node_to_string(const TemplateNode &n) {
     if (n.col_relative == 1) s += "col_index_relative:1\n";  // not upstream keys
     if (n.col_relative == 2) s += "col_index_diagonal:1\n";
     if (n.col_relative == 3) s += "col_index_runs:1\n";
+    if (n.own_rows == 1) s += "y_rows_owned:1\n";
     // upstream closes every kernel node with one more "}" than it opened (exe_graph.cc:3547); kept,
     // since readers of test.log are written against that text
     return s + "}\n}\n";
@@ -399,6 +400,34 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
           c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
                 " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
                 " column runs -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
+          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+        }
+      } catch (const std::exception &e) {
+        c.res.failed_candidates++;
+        c.log(std::string("  candidate failed: ") + e.what());
+      }
+      // and the best of the two once more under row ownership (whole row groups per workgroup, rows stored
+      // without atomics, no clear of y), where the sub-matrix allows it
+      try {
+        add_template_to_builder(*b, sub, type);
+        compress_template_in_builder(*b, sub);
+        if (best.col_relative == 3) AS_CHECK(set_column_runs(*b, sub), "column runs cannot be rebuilt");
+        if (set_row_ownership(*b, sub)) {
+          load_and_upload(*b, c.opt.device);
+          if (as_hip_h2d(b->x.ptr, c.probe_x.data(), b->x.bytes) != 0) throw Error(as_hip_last_error());
+          TemplateNode n = best;
+          n.own_rows = 1;
+          n.tblock_num = 0;  // one workgroup per trip of the new form
+          set_launch(*b->subs[sub].tpl, n);
+          invalidate_module(*b);
+          verify_candidate(c, *b, m, (int64_t)sub);
+          float ms = 0, gf = 0;
+          time_builder(c, *b, ms, gf);
+          c.res.candidates++;
+          n.tblock_num = (long)b->subs[sub].tpl->tblock_num;
+          c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
+                " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
+                " row ownership -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
           if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
         }
       } catch (const std::exception &e) {
@@ -843,6 +872,8 @@ BuiltGraph build_from_graph(const CooInput &in, const BestGraph &g, unsigned wav
       AS_CHECK(set_diagonal_columns(*r.builder, s), "the best graph's diagonal columns cannot be rebuilt");
     if (g.subs[s].tpl.col_relative == 3)
       AS_CHECK(set_column_runs(*r.builder, s), "the best graph's column runs cannot be rebuilt");
+    if (g.subs[s].tpl.own_rows == 1)
+      AS_CHECK(set_row_ownership(*r.builder, s), "the best graph's row ownership cannot be rebuilt");
     set_launch(*r.builder->subs[s].tpl, g.subs[s].tpl);
   }
   return r;

@@ -54,6 +54,8 @@ struct TemplateNode {
   // slot's diagonal, no column array (set_diagonal_columns); 3: tile template in its column-run form
   // (set_column_runs)
   long col_relative = 0;
+  // 1: tile template under row ownership (set_row_ownership)
+  long own_rows = 0;
 };
 std::string convert_template_node_to_string(const TemplateNode &n);   // exe_graph.cc:3317
 

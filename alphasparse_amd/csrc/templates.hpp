@@ -80,6 +80,10 @@ struct Template {
   // of consecutive columns plus a byte of run starts (no upstream counterpart; dense blocks, dense rows): see
   // init_tile_template_with_column_runs
   bool col_runs = false;
+  // tile template: every row group belongs to one workgroup, which keeps the group's row sums in LDS across the
+  // slices and stores the rows to y at the end -- no atomics, no clear of y (no upstream counterpart; matrices of
+  // many row groups that meet few slices each): see init_tile_template_variant
+  bool own_rows = false;
   // LDS the kernel asks for at launch (beyond its static __shared__ arrays)
   uint64_t dynamic_lds_bytes = 0;
   // Device scratch of the kernels (last argument `scratch_arr`): allocated and cleared once at upload; what
@@ -153,6 +157,10 @@ bool make_columns_diagonal(Template &t);
 // lane that would hold more than four runs is closed with zero-valued elements, so the form exists for every
 // matrix the template supports, and costs padding where columns are not consecutive: compare val_arr sizes.
 std::unique_ptr<Template> init_tile_template_with_column_runs(const Matrix &m, uint64_t sub);
+// SHARED_MEMORY_TILE_TEMPLATE in any combination of its two forms (column runs, row ownership); nullptr when row
+// ownership is asked for and does not fit the sub-matrix: a column band of the matrix, slice copies that would
+// move more than a quarter of the element stream's bytes, or trips (whole row groups) too uneven to fill the device.
+std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows);
 // HIP source of `extern "C" __global__ void spmv_<sub>(...)`.
 std::string code_of_template_kernal(const Template &t);
 // Kernel arguments in order: names of the metadata arrays that are passed

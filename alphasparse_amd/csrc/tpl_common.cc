@@ -103,6 +103,8 @@ bool template_needs_cleared_y(const Template &t, const Matrix &m, uint64_t sub) 
   // the two-kernel LDS templates store every row of the strip in their finish kernel, with or without elements
   if (t.finish_tblock_num && (t.type == SHARED_MEMORY_TILE_TEMPLATE || t.type == SHARED_MEMORY_PRODUCT_BIN_TEMPLATE))
     return false;
+  // the tile template under row ownership stores every row of every row group, zeros included
+  if (t.type == SHARED_MEMORY_TILE_TEMPLATE && t.own_rows) return false;
   // the row-wise templates store the rows that have a unit (TLB, WLB or BLB): a row without elements has none
   const DenseItem &it = m.items[sub];
   const uint64_t sub_rows = it.max_row - it.min_row + 1;
@@ -161,6 +163,11 @@ namespace tpl_shared_memory_tile { std::unique_ptr<Template> init_with_column_ru
 std::unique_ptr<Template> init_tile_template_with_column_runs(const Matrix &m, uint64_t sub) {
   AS_CHECK(is_supported_by_template(SHARED_MEMORY_TILE_TEMPLATE, m, sub), "format is not supported by SHARED_MEMORY_TILE_TEMPLATE");
   return tpl_shared_memory_tile::init_with_column_runs(m, sub);
+}
+namespace tpl_shared_memory_tile { std::unique_ptr<Template> init_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows); }
+std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows) {
+  AS_CHECK(is_supported_by_template(SHARED_MEMORY_TILE_TEMPLATE, m, sub), "format is not supported by SHARED_MEMORY_TILE_TEMPLATE");
+  return tpl_shared_memory_tile::init_variant(m, sub, column_runs, own_rows);
 }
 std::string code_of_template_kernal(const Template &t) { AS_DISPATCH(t.type, kernel_source(t)) }
 

@@ -63,11 +63,15 @@ bool is_supported(const Matrix &m, uint64_t sub) {
   return true;
 }
 
-static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs);
-std::unique_ptr<Template> init(const Matrix &m, uint64_t sub) { return build(m, sub, false); }
-std::unique_ptr<Template> init_with_column_runs(const Matrix &m, uint64_t sub) { return build(m, sub, true); }
+static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows);
+std::unique_ptr<Template> init(const Matrix &m, uint64_t sub) { return build(m, sub, false, false); }
+std::unique_ptr<Template> init_with_column_runs(const Matrix &m, uint64_t sub) { return build(m, sub, true, false); }
+// nullptr when row ownership does not fit the sub-matrix (see build)
+std::unique_ptr<Template> init_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows) {
+  return build(m, sub, column_runs, own_rows);
+}
 
-static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs) {
+static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows) {
   AS_CHECK(is_supported(m, sub), "format is not supported by SHARED_MEMORY_TILE_TEMPLATE");
   const DenseItem &it = m.items[sub];
   const CompressedBlock &cb = *it.cb;
@@ -98,13 +102,71 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   // one trip per workgroup the 256 CUs hold at a time with this much LDS each
   uint64_t want = kCuNum * std::max<uint64_t>(1, kLdsBytes / ((S + R) * vs));
   want = std::max<uint64_t>(1, std::min<uint64_t>(want, (n + 16383) / 16384));
+  std::vector<uint64_t> group_first_block{0};
+  // Row ownership (own_rows): the BLBs are taken row group by row group (inside a row group slice by slice) and
+  // a trip is a whole number of row groups, so that one workgroup holds every sum of its rows: the cells of a row
+  // group live in LDS across its slices, a cell is the row's place in the group, and at the end of the group the
+  // rows are STORED to y -- no atomics, no table of places, y needs no clear.  The price is one slice copy per
+  // (row group, slice) tile instead of one per trip and slice, and trips as coarse as row groups: the form is
+  // turned down (nullptr) where the copies would move more than a quarter of the element stream's bytes, where
+  // there are fewer trips than half the workgroups the device holds, or where the heaviest trip would take more
+  // than 1.2 times the average.  It fits matrices of many row groups that meet few
+  // slices each (banded matrices); strips of a few very long rows stay with the slice-by-slice order.
+  std::vector<uint64_t> blk_order(B), trip_first_row_group;
+  for (uint64_t b = 0; b < B; b++) blk_order[b] = b;
+  if (own_rows) {
+    if (sub_block_is_col_restricted(m, sub)) return nullptr;  // another sub-matrix adds to the same rows
+    std::stable_sort(blk_order.begin(), blk_order.end(), [&](uint64_t x, uint64_t y) {
+      return blk_rg[x] != blk_rg[y] ? blk_rg[x] < blk_rg[y] : blk_slice[x] < blk_slice[y];
+    });
+    const uint64_t NG = (sub_rows + R - 1) / R;
+    std::vector<uint64_t> group_cost(NG, 0);
+    uint64_t tiles = 0, stream_cost = 0;
+    for (uint64_t i = 0; i < B; i++) {
+      const uint64_t b = blk_order[i];
+      group_cost[blk_rg[b]] += blk_cost[b];
+      stream_cost += blk_cost[b];
+      if (i == 0 || blk_rg[b] != blk_rg[blk_order[i - 1]] || blk_slice[b] != blk_slice[blk_order[i - 1]]) {
+        group_cost[blk_rg[b]] += slice_cost;
+        tiles++;
+      }
+    }
+    if (tiles * slice_cost * 4 > stream_cost) return nullptr;
+    uint64_t total = 0;
+    for (uint64_t c : group_cost) total += c;
+    // as many trips as workgroups fit, or the fewest more row groups per trip that make the trips even
+    const uint64_t groups_per_trip = (NG + want - 1) / want;
+    const uint64_t trips = (NG + groups_per_trip - 1) / groups_per_trip, per_trip = total / trips + 1;
+    uint64_t cost = 0, heaviest = 0;
+    trip_first_row_group.push_back(0);
+    for (uint64_t g = 0; g < NG; g++) {
+      if (cost > 0 && cost + group_cost[g] / 2 > per_trip && trip_first_row_group.size() < trips) {
+        heaviest = std::max(heaviest, cost);
+        trip_first_row_group.push_back(g);
+        cost = 0;
+      }
+      cost += group_cost[g];
+    }
+    heaviest = std::max(heaviest, cost);
+    trip_first_row_group.push_back(NG);
+    const uint64_t T = trip_first_row_group.size() - 1;
+    // too few trips leave most CUs idle; uneven trips make the others wait for the heaviest
+    if (T * 2 < want || heaviest * T * 10 > total * 12) return nullptr;
+    // BLB view of the trips, in the order of blk_order
+    group_first_block.clear();
+    uint64_t i = 0;
+    for (uint64_t tp = 0; tp < T; tp++) {
+      group_first_block.push_back(i);
+      while (i < B && blk_rg[blk_order[i]] < trip_first_row_group[tp + 1]) i++;
+    }
+    group_first_block.push_back(B);
+  } else {
   uint64_t total_cost = want * slice_cost;
   for (uint64_t b = 0; b < B; b++) {
     total_cost += blk_cost[b];
     if (b == 0 || blk_slice[b] != blk_slice[b - 1]) total_cost += slice_cost;
   }
   const uint64_t per_group = total_cost / want + 1;
-  std::vector<uint64_t> group_first_block{0};
   {
     uint64_t cost = 0;
     for (uint64_t b = 0; b < B; b++) {
@@ -120,8 +182,10 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     }
     group_first_block.push_back(B);
   }
+  }
   const uint64_t G = group_first_block.size() - 1;
   t->scalar["group_num"] = G;
+  t->own_rows = own_rows;
 
   // y row of every row of the sub-matrix (through the sort permutation when there is one)
   std::vector<uint64_t> y_row(sub_rows);
@@ -131,7 +195,9 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   // row of the strip touches costs a trip to memory.  The sums are then collected in a dense
   // scratch vector (one value per row of the strip) and moved to y by spmv_<sub>_finish, with plain
   // stores: the rows of a row strip belong to this kernel alone.
-  if (t->global_sort_index && !sub_block_is_col_restricted(m, sub)) {
+  if (own_rows) {
+    t->is_atom_add = false;  // every row is stored once, by the workgroup that owns its row group
+  } else if (t->global_sort_index && !sub_block_is_col_restricted(m, sub)) {
     t->scratch_bytes = sub_rows * vs;
     t->scratch_starts_zero = true;  // row sums are added into it; the finish kernel leaves it cleared
     t->is_atom_add = false;  // y itself is written once, by the finish kernel
@@ -141,8 +207,11 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   const uint64_t y_base = !t->global_sort_index ? t->kernal_first_row_index : 0;
   auto target_of = [&](uint64_t sub_row) { return t->scratch_bytes ? sub_row : y_row[sub_row] + y_base; };
 
-  // runs: maximal sequences of BLBs of one tile inside a trip, padded to kRunUnit elements
-  std::vector<uint64_t> group_first_run, run_slice, run_nz_begin{0}, run_piece_begin{0}, piece_target;
+  // runs: maximal sequences of BLBs of one tile inside a trip, padded to kRunUnit elements.  A piece is numbered
+  // by its order inside the run -- or, under row ownership, by the row's place in its row group, which every run
+  // of the group shares; a lane's pieces must then still be consecutive numbers, so where a row of the group has
+  // no element in the slice the lane is closed with zero-valued elements and the next row opens a new lane.
+  std::vector<uint64_t> group_first_run, run_slice, run_nz_begin{0}, run_piece_begin{0}, piece_target, run_row_group;
   std::vector<uint64_t> lcol, piece;  // per element: column inside the slice, piece number inside the run
   uint64_t lane_runs = 0;             // column-run form: runs of consecutive columns in the lane being filled
   lcol.reserve(n + G * kRunUnit);
@@ -150,13 +219,18 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   t->val_arr.reserve(n + G * kRunUnit);
   for (uint64_t g = 0; g < G; g++) {
     group_first_run.push_back(run_slice.size());
-    uint64_t b = group_first_block[g], b_end = group_first_block[g + 1];
-    while (b < b_end) {
-      uint64_t e = b;
-      while (e < b_end && blk_slice[e] == blk_slice[b] && blk_rg[e] == blk_rg[b]) e++;
-      const uint64_t col0 = blk_slice[b] * S, k0 = bl.coo_begin[b], k1 = bl.coo_begin[e];
+    uint64_t i = group_first_block[g], i_end = group_first_block[g + 1];
+    while (i < i_end) {
+      const uint64_t b = blk_order[i];
+      uint64_t e = i;
+      while (e < i_end && blk_slice[blk_order[e]] == blk_slice[b] && blk_rg[blk_order[e]] == blk_rg[b]) {
+        AS_CHECK(e == i || blk_order[e] == blk_order[e - 1] + 1, "the BLBs of a tile must follow each other");
+        e++;
+      }
+      const uint64_t col0 = blk_slice[b] * S, k0 = bl.coo_begin[b], k1 = bl.coo_begin[blk_order[e - 1] + 1];
       const uint64_t slice_len = std::min<uint64_t>(S, t->matrix_cols - t->kernal_first_col_index - col0);
-      uint64_t pieces = 0;
+      const uint64_t row0 = blk_rg[b] * R;
+      uint64_t pieces = 0, cur_piece = 0;
       // a zero-valued element on the current piece; in the column-run form its column continues the run where
       // that stays inside the slice, and otherwise opens a run at column 0
       auto pad = [&]() {
@@ -164,11 +238,15 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
         if (column_runs && lcol.size() % kLaneElems != 0 && lcol.back() + 1 < slice_len) c = lcol.back() + 1;
         else if (column_runs) lane_runs++;
         lcol.push_back(c);
-        piece.push_back(pieces - 1);
+        piece.push_back(cur_piece);
         t->val_arr.push_back(0.0);
       };
       for (uint64_t k = k0; k < k1; k++) {
         const uint64_t c = col[k] - col0;
+        const bool new_row = k == k0 || row[k] != row[k - 1];
+        // row ownership: a row that does not follow its predecessor directly cannot share a lane with it
+        if (own_rows && new_row && k != k0 && row[k] != row[k - 1] + 1)
+          while (lcol.size() % kLaneElems) pad();
         if (column_runs) {
           if (lcol.size() % kLaneElems == 0) lane_runs = 0;
           if (lcol.size() % kLaneElems == 0 || c != lcol.back() + 1) {
@@ -179,23 +257,25 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
             lane_runs++;
           }
         }
-        if (k == k0 || row[k] != row[k - 1]) {
-          piece_target.push_back(target_of(row[k]));
+        if (new_row) {
+          if (!own_rows) piece_target.push_back(target_of(row[k]));
           pieces++;
+          cur_piece = own_rows ? row[k] - row0 : pieces - 1;
         }
         lcol.push_back(c);
-        piece.push_back(pieces - 1);
+        piece.push_back(cur_piece);
         t->val_arr.push_back(val[k]);
       }
-      AS_CHECK(pieces <= R, "more row pieces in a run than rows in a row group");
+      AS_CHECK(pieces <= R && cur_piece < R, "more row pieces in a run than rows in a row group");
       while (lcol.size() % kRunUnit) {
         if (column_runs && lcol.size() % kLaneElems == 0) lane_runs = 0;
         pad();
       }
       run_slice.push_back(blk_slice[b]);
+      run_row_group.push_back(blk_rg[b]);
       run_nz_begin.push_back(lcol.size() / kRunUnit);
       run_piece_begin.push_back(piece_target.size());
-      b = e;
+      i = e;
     }
   }
   group_first_run.push_back(run_slice.size());
@@ -220,7 +300,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     };
     for (uint64_t run = 0; run < run_slice.size(); run++) {
       const uint64_t p0 = run_nz_begin[run] * kRunUnit, p1 = run_nz_begin[run + 1] * kRunUnit;
-      sums_of_piece.assign(run_piece_begin[run + 1] - run_piece_begin[run], 0);
+      sums_of_piece.assign(own_rows ? R : run_piece_begin[run + 1] - run_piece_begin[run], 0);
       for (uint64_t at = p0; at < p1; at += kLaneElems) {
         uint64_t w = piece[at];
         for (uint64_t j = 1; j < kLaneElems; j++) {
@@ -278,8 +358,12 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   add("group_first_run", std::move(group_first_run), true);
   add("run_slice", std::move(run_slice), true);
   add("run_nz_begin", std::move(run_nz_begin), true);
-  add("run_piece_begin", std::move(run_piece_begin), true);
-  add("piece_target", std::move(piece_target), true);
+  if (own_rows) {
+    add("run_row_group", std::move(run_row_group), true);
+  } else {
+    add("run_piece_begin", std::move(run_piece_begin), true);
+    add("piece_target", std::move(piece_target), true);
+  }
   add("lane_word", std::move(lane_word), true);
   if (column_runs) {
     TArr a;
@@ -288,17 +372,22 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     t->arrays.push_back(std::move(a));
   }
   add("y_row_index", std::move(y_row), false);
-  t->find("y_row_index")->on_device = t->finish_tblock_num != 0;  // the finish kernel's map; the main kernel has piece_target
+  // the finish kernel's map (the main kernel has piece_target), or the map of the rows a workgroup owns
+  t->find("y_row_index")->on_device = t->finish_tblock_num != 0 || (own_rows && t->global_sort_index);
   add("group_first_block", std::move(group_first_block), false);  // BLB view of the trips, host only
   t->find("group_first_block")->on_device = false;
+  if (own_rows) {
+    add("trip_first_row_group", std::move(trip_first_row_group), false);  // host only
+    t->find("trip_first_row_group")->on_device = false;
+  }
   tpl_shared_memory_tile::set_default_launch(*t);
   return t;
 }
 
 void try_all_compress(Template &t) {
-  for (const char *name : {"group_first_run", "run_slice", "run_nz_begin", "run_piece_begin", "y_row_index"}) {
-    TArr &a = *t.find(name);
-    if (!a.c.active()) init_linear_compressor(a.a, a.c, true);
+  for (const char *name : {"group_first_run", "run_slice", "run_nz_begin", "run_piece_begin", "run_row_group", "y_row_index"}) {
+    TArr *a = t.find(name);
+    if (a && !a->c.active()) init_linear_compressor(a->a, a->c, true);
   }
 }
 
@@ -310,7 +399,8 @@ void set_default_launch(Template &t) {
 
 std::string kernel_source(const Template &t) {
   const std::string vt = value_type_name(t);
-  AS_CHECK(t.col_index_arr.dt == UNSIGNED_SHORT && t.arr("lane_word").a.dt == UNSIGNED_INT && t.arr("piece_target").a.dt == UNSIGNED_INT,
+  AS_CHECK(t.col_index_arr.dt == UNSIGNED_SHORT && t.arr("lane_word").a.dt == UNSIGNED_INT &&
+               (t.own_rows || t.arr("piece_target").a.dt == UNSIGNED_INT),
            "slice columns must be 16 bits wide, lane words and piece targets 32");
   AS_CHECK(t.thread_num_in_block % 64 == 0 && t.thread_num_in_block >= 64 && t.thread_num_in_block <= 1024,
            "thread_num_in_block must be a multiple of 64 up to 1024");
@@ -349,16 +439,21 @@ std::string kernel_source(const Template &t) {
   s += "    run_begin = __builtin_amdgcn_readfirstlane(run_begin); run_end = __builtin_amdgcn_readfirstlane(run_end);\n";
   s += "    __syncthreads();\n";  // the previous trip's write-back is done with the cells
   s += "    for (unsigned int i = threadIdx.x; i < " + Rs + "; i += " + B + ") piece_sum[i] = 0;\n";
-  s += "    unsigned int cur_slice = 0xffffffffu, done_begin = 0u, done_end = 0u;\n";
+  if (t.own_rows) s += "    unsigned int cur_slice = 0xffffffffu, cur_group = 0xffffffffu;\n";
+  else s += "    unsigned int cur_slice = 0xffffffffu, done_begin = 0u, done_end = 0u;\n";
   s += "    for (unsigned int run = run_begin; run <= run_end; run++)\n    {\n";
   // run == run_end is the write-back of the trip's last run
-  s += "      unsigned int next_run = run + 1u, slice = 0xffffffffu, unit_begin = 0u, unit_end = 0u, piece_begin = 0u, piece_end = 0u;\n";
+  s += "      unsigned int next_run = run + 1u, slice = 0xffffffffu, unit_begin = 0u, unit_end = 0u, piece_begin = 0u, piece_end = 0u, row_group = 0xffffffffu;\n";
   s += "      if (run < run_end)\n      {\n";
   s += "        " + code_of_meta_read(t, "run_slice", "slice", "run");
   s += "        " + code_of_meta_read(t, "run_nz_begin", "unit_begin", "run");
   s += "        " + code_of_meta_read(t, "run_nz_begin", "unit_end", "next_run");
-  s += "        " + code_of_meta_read(t, "run_piece_begin", "piece_begin", "run");
-  s += "        " + code_of_meta_read(t, "run_piece_begin", "piece_end", "next_run");
+  if (t.own_rows) {
+    s += "        " + code_of_meta_read(t, "run_row_group", "row_group", "run");
+  } else {
+    s += "        " + code_of_meta_read(t, "run_piece_begin", "piece_begin", "run");
+    s += "        " + code_of_meta_read(t, "run_piece_begin", "piece_end", "next_run");
+  }
   s += "      }\n";
   s += "      __syncthreads();\n";  // every wavefront is done with the previous run
   // Between two runs a workgroup writes the finished run back (a table read and one atomic per piece) and, when the
@@ -370,6 +465,23 @@ std::string kernel_source(const Template &t) {
   // requests a batch of loads before it stores the first.
   const uint64_t wb_batch = std::min<uint64_t>(kBetweenRunsBatch, std::max<uint64_t>(1, (R + t.thread_num_in_block - 1) / t.thread_num_in_block));
   const std::string Ws = std::to_string(wb_batch);
+  if (t.own_rows) {
+    // Row ownership: a row group's cells stay in LDS across its runs (one per slice it meets); when the coming run
+    // belongs to another row group -- or the trip ends -- the finished group's rows are stored to y, zeros for rows
+    // without elements included: no other workgroup holds a sum of these rows.
+    const std::string y_off = (!t.global_sort_index && t.kernal_first_row_index != 0 ? " + " + std::to_string(t.kernal_first_row_index) + "u" : std::string());
+    s += "      if (row_group != cur_group)\n      {\n";
+    s += "        if (cur_group != 0xffffffffu)\n        {\n";
+    s += "          const unsigned int row0 = cur_group * " + Rs + ", live = min(" + Rs + ", " + std::to_string(rows) + "u - row0);\n";
+    s += "          for (unsigned int i = threadIdx.x; i < live; i += " + B + ")\n          {\n";
+    s += "            const " + vt + " sum = piece_sum[i];\n            piece_sum[i] = 0;\n";
+    s += "            const unsigned int sub_row = row0 + i;\n            unsigned int global_row_index;\n";
+    if (t.global_sort_index) s += "            " + code_of_meta_read(t, "y_row_index", "global_row_index", "sub_row");
+    else s += "            global_row_index = sub_row;\n";
+    s += "            as_stnt(device_y_arr + global_row_index" + y_off + ", sum);\n";
+    s += "          }\n        }\n";
+    s += "        cur_group = row_group;\n      }\n";
+  } else {
   // write-back of the run that ended: consecutive lanes take consecutive pieces (rows in rising order)
   s += "      for (unsigned int i0 = threadIdx.x; i0 < done_end - done_begin; i0 += " + B + " * " + Ws + "u)\n      {\n";
   s += "        typedef __attribute__((address_space(1))) " + vt + " *global_ptr_t;\n";
@@ -389,6 +501,7 @@ std::string kernel_source(const Template &t) {
   s += "          if (sum[j] != 0) __builtin_amdgcn_global_atomic_fadd_" + std::string(t.val_dtype == DOUBLE ? "f64" : "f32") + "(where[j], sum[j]);\n";
   s += "      }\n";
   s += "      done_begin = piece_begin; done_end = piece_end;\n";
+  }
   s += "      if (run < run_end && slice != cur_slice)\n      {\n";
   s += "        const unsigned int col0 = slice * " + Ss + ";\n";
   s += "        const unsigned int slice_len = min(" + Ss + ", " + std::to_string(x_len) + "u - col0);\n";
@@ -460,7 +573,9 @@ std::string kernel_source(const Template &t) {
   // is the only one of its piece before the write-back: a plain store will do.
   auto emit = [&](unsigned j) {
     const std::string bit = std::to_string(1u << (kStoreBit + j)) + "u";
-    return "{ if (w[k] & " + bit + ") piece_sum[cell] = acc; else as_lds_add(piece_sum + cell, acc); }";
+    // under row ownership a cell may hold the row's sum from an earlier slice: the only sum of its piece IN THIS
+    // RUN is added without an atomic (nobody else touches the cell before the next barrier)
+    return "{ if (w[k] & " + bit + ") piece_sum[cell] " + std::string(t.own_rows ? "+=" : "=") + " acc; else as_lds_add(piece_sum + cell, acc); }";
   };
   s += "          unsigned int cell = w[k] & 0x7fffu;\n";
   s += "          " + vt + " acc = a[k][0][0] * xv[0];\n";

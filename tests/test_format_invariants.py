@@ -183,9 +183,21 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
     added: y comes out right only if every flagged piece gets that one sum."""
     arr = {k: np.asarray(a[0]).astype(np.int64) for k, a in t["arrays"].items()}
     val = np.asarray(t["val_arr"][0] if isinstance(t["val_arr"], tuple) else t["val_arr"], np.float64)
-    gfr, rs, nzb, rpb, target, word, yrow, lcol = (arr["group_first_run"], arr["run_slice"], arr["run_nz_begin"],
-                                                   arr["run_piece_begin"], arr["piece_target"], arr["lane_word"],
-                                                   arr["y_row_index"], arr["col_index_arr"])
+    own_rows = "run_row_group" in arr   # row ownership: cells are rows of the run's row group, kept across its runs
+    gfr, rs, nzb, word, yrow, lcol = (arr["group_first_run"], arr["run_slice"], arr["run_nz_begin"], arr["lane_word"],
+                                      arr["y_row_index"], arr["col_index_arr"])
+    if own_rows:
+        rrg = arr["run_row_group"]
+        assert "piece_target" not in arr and "run_piece_begin" not in arr and len(rrg) == len(rs)
+        # a trip is a whole number of row groups, a row group the runs of one trip that follow each other
+        trip_of_run = np.repeat(np.arange(len(gfr) - 1), np.diff(gfr))
+        for g in np.unique(rrg):
+            runs = np.flatnonzero(rrg == g)
+            assert (np.diff(runs) == 1).all() and len(set(trip_of_run[runs].tolist())) == 1
+            assert (np.diff(rs[runs]) > 0).all()                 # slice by slice inside the group
+        assert (np.diff(rrg) >= 0).all()
+    else:
+        rpb, target = arr["run_piece_begin"], arr["piece_target"]
     if "col_run_mask" in arr:
         # column-run form: per lane the first columns of up to four runs of consecutive columns and a byte whose
         # bit j says that element j opens the next run (a run beyond the fourth starts at column 0)
@@ -201,8 +213,10 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
         lcol = decoded.reshape(-1)
     assert gfr[0] == 0 and gfr[-1] == len(rs) and (np.diff(gfr) > 0).all() and (np.diff(nzb) > 0).all()
     assert nzb[-1] * 512 == len(lcol) == len(val) == 8 * len(word) and (lcol < slice_width).all()
-    assert rpb[0] == 0 and rpb[-1] == len(target) and (np.diff(rpb) > 0).all() and (np.diff(rpb) <= group).all()
-    through_scratch = t["scalars"]["is_atom_add"] == 0
+    if not own_rows:
+        assert rpb[0] == 0 and rpb[-1] == len(target) and (np.diff(rpb) > 0).all() and (np.diff(rpb) <= group).all()
+    through_scratch = t["scalars"]["is_atom_add"] == 0 and not own_rows
+    group_cells = {}
     # values are stored 16 bytes per lane and load: piece i of lane l of a wavefront step at (i * 64 + l)
     j, lane = np.meshgrid(np.arange(8), np.arange(64))
     where = ((j // chunk) * 64 + lane) * chunk + j % chunk       # [lane, j] -> place inside the step
@@ -211,7 +225,10 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
     flagged = plain = 0
     for run in range(len(rs)):
         k0, k1 = nzb[run] * 512, nzb[run + 1] * 512
-        cells = np.zeros(rpb[run + 1] - rpb[run])
+        if own_rows:
+            cells = group_cells.setdefault(int(rrg[run]), np.zeros(group))
+        else:
+            cells = np.zeros(rpb[run + 1] - rpb[run])
         touched = np.zeros(len(cells), np.int64)
         prod = val[k0:k1] * x[rs[run] * slice_width + lcol[k0:k1]]
         for u in range(0, k1 - k0, 512):                         # one wavefront step
@@ -221,7 +238,10 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
             store = (w[:, None] >> (22 + np.arange(8))[None, :]) & 1
             final = first + new_piece.sum(1)
             step = first[1:] - final[:-1]
-            assert ((step == 0) | (step == 1)).all()              # the next lane goes on with the piece or starts the next one
+            if own_rows:
+                assert (step >= 0).all()                         # a lane may skip rows that have no element in the slice
+            else:
+                assert ((step == 0) | (step == 1)).all()          # the next lane goes on with the piece or starts the next one
             carry = 0.0                                          # the segmented sum over the lanes' last pieces
             for lane in range(64):
                 cell, acc = first[lane], 0.0
@@ -230,8 +250,8 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
                     nonlocal flagged, plain
                     assert cell < len(cells)
                     if store[lane, j]:
-                        assert touched[cell] == 0                # the only sum of this piece
-                        cells[cell] = acc
+                        assert touched[cell] == 0                # the only sum of this piece (in this run)
+                        cells[cell] = cells[cell] + acc if own_rows else acc
                         touched[cell] = -1
                         flagged += 1
                     else:
@@ -251,9 +271,19 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
                     carry = 0.0
                 else:
                     carry = acc
+        if own_rows:
+            continue
         assert (touched != 0).all()                              # every piece of the run got a sum
         rows_of_run = target[rpb[run]:rpb[run + 1]]
         np.add.at(y, yrow[rows_of_run] if through_scratch else rows_of_run, cells)
+    if own_rows:
+        # every row of every row group is stored once, rows without elements as zeros; a row group that holds no
+        # element at all belongs to no run: its rows are... not written (there is none in a matrix without empty rows)
+        y[:] = np.nan
+        for g, cells in group_cells.items():
+            live = min(group, sub_rows - g * group)
+            y[yrow[g * group:g * group + live]] = cells[:live]
+        assert not np.isnan(y).any()
     return y, flagged, plain
 
 
@@ -303,6 +333,75 @@ def test_tile_division_and_tile_template(slice_width, group, blb, sort):
             assert t["arrays"]["col_index_arr"][1] == "UNSIGNED_SHORT" and t["arrays"]["lane_word"][1] == "UNSIGNED_INT"
     src = b.kernel_source()
     assert "as_wave_segmented_sum" in src and ("y_row_index[" in src) == sort
+
+
+@pytest.mark.parametrize("vdt,chunk", [(K.FLOAT, 4), (K.DOUBLE, 2)], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("sort,runs", [(False, False), (True, False), (False, True), (True, True)],
+                         ids=["plain", "sorted", "plain_runs", "sorted_runs"])
+def test_tile_template_under_row_ownership(vdt, chunk, sort, runs):
+    """set_row_ownership on a banded matrix of dense 3 x 3 blocks (many row groups, two or three slices each): the
+    tiles row group by row group, cells = rows of the group kept across its slices, lanes closed where a row of the
+    group is missing from a slice, no piece tables, no scratch, no atomics into y -- and the same y when the arrays
+    are walked the way the kernel walks them, alone and on top of the column-run form.  Turned down where it does
+    not fit: a few long rows (one row group for all CUs), a column band, another template."""
+    from alphasparse_amd import skeletons as SK
+    rows, cols, r, c, v, x = S.fem_blocks(1000, 27, 60, seed=5)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    if sort:
+        m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+    m.execute_strategy(K.COMPRESS_NONE)
+    tp = SK.apply_skeleton(m, 0, "T1", slice=500, group=100, b=1000)[0]
+    b = A.Builder(m)
+    b.set_template(0, tp, compress=False)
+    b.set_launch(0, thread_num_in_block=256)
+    if runs:
+        assert b.set_column_runs(0)
+    before = b.template_dump(0)
+    assert b.clears_y() == (not sort)                                    # atomics into y, or the scratch vector
+    assert b.set_row_ownership(0) and not b.set_row_ownership(0)         # the second call finds the form in place
+    t = b.template_dump(0)
+    assert 0.95 * len(before["val_arr"]) <= len(t["val_arr"]) <= 1.05 * len(before["val_arr"])   # other runs, other padding
+    assert ("col_run_mask" in t["arrays"]) == runs and "run_row_group" in t["arrays"]
+    assert t["scalars"]["is_atom_add"] == 0 and not b.clears_y()
+    assert b.get_launch(0)["thread_num_in_block"] == 256
+    vv = np.float32(v).astype(np.float64) if vdt == K.FLOAT else v.astype(np.float64)
+    yref = np.zeros(rows)
+    np.add.at(yref, np.asarray(r, np.int64), vv * x[np.asarray(c, np.int64)])
+    y, flagged, plain = _emulate_tile_template(t, 500, 100, rows, x.astype(np.float64), chunk=chunk)
+    assert np.allclose(y, yref, rtol=1e-12, atol=1e-12) and flagged > 0
+    src = b.kernel_source()
+    assert "cur_group" in src and "piece_target" not in src and "_finish" not in src and ("y_row_index[" in src) == sort
+    assert ("col_run_mask" in src) == runs
+    # the column-run form on top of row ownership keeps the ownership
+    if not runs:
+        assert b.set_column_runs(0)
+        t2 = b.template_dump(0)
+        assert "run_row_group" in t2["arrays"] and "col_run_mask" in t2["arrays"]
+        y2 = _emulate_tile_template(t2, 500, 100, rows, x.astype(np.float64), chunk=chunk)[0]
+        assert np.allclose(y2, yref, rtol=1e-12, atol=1e-12)
+    # a few long rows: one row group would have to feed every CU
+    rows, cols, r, c, v, x = cases._steps([30000] * 6, 40000, 4)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    m.execute_strategy(K.COMPRESS_NONE)
+    b = A.Builder(m)
+    b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=512, group=64, b=4096)[0])
+    assert not b.set_row_ownership(0) and "run_row_group" not in b.template_dump(0)["arrays"]
+    # a column band of the matrix shares its rows with the other bands
+    rows, cols, r, c, v, x = S.fem_blocks(400, 9, 60, seed=5)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    m.execute_node(K.DENSE_FIXED_COL_DIV, -1, scalars=(600,))
+    m.execute_strategy(K.COMPRESS_NONE)
+    for sub in range(m.info()["n_sub"]):
+        tp = SK.apply_skeleton(m, sub, "T1", slice=500, group=64, b=1000)[0]
+    b = A.Builder(m)
+    b.set_template(0, tp)
+    assert not b.set_row_ownership(0)
+    # another template
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    m.execute_strategy(K.COMPRESS_NONE)
+    b = A.Builder(m)
+    b.set_template(0, SK.apply_skeleton(m, 0, "S1", m=64)[0])
+    assert not b.set_row_ownership(0)
 
 
 def test_tile_template_stores_fp64_values_two_per_lane_and_load():

@@ -309,6 +309,41 @@ def test_tile_template_in_column_run_form(gpu, vdt, sort, threads):
         b.close()
 
 
+@pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("sort", [False, True], ids=["plain", "sorted"])
+@pytest.mark.parametrize("runs", [False, True], ids=["columns", "runs"])
+@pytest.mark.parametrize("threads", [1024, 256])
+def test_tile_template_under_row_ownership(gpu, vdt, sort, runs, threads):
+    """The tile kernel with whole row groups per workgroup (rows stored to y, no atomics, no clear): same y as the CPU
+    CSR oracle on banded matrices of dense 3 x 3 blocks (row groups that meet two or three slices, a last slice and
+    a last row group shorter than the others, rows at the ragged edge of the band that miss a slice of their group:
+    lanes closed where the next row of the group has no element in the slice); y holds NaN before the call."""
+    for gen, slice_width, group in ((lambda: S.fem_blocks(3000, 27, 400), 4000, 250), (lambda: S.fem_blocks(1000, 9, 60, seed=3), 500, 100),
+                                    (lambda: S.fem_blocks(2000, 27, 100, seed=9), 1000, 120)):
+        rows, cols, r, c, v, x = gen()
+        npd = NP[vdt]
+        v, x = v.astype(npd), x.astype(npd)
+        y_ref, mag = oracle_y(rows, r, c, v, x)
+        m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+        if sort:
+            m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+        m.execute_strategy(K.COMPRESS_NONE)
+        tp = SK.apply_skeleton(m, 0, "T1", slice=slice_width, group=group, b=4096)[0]
+        b = A.Builder(m)
+        b.set_template(0, tp)
+        if runs and not b.set_column_runs(0):
+            b.close()
+            continue                                             # scattered columns: the column-run form is turned down
+        assert b.set_row_ownership(0), (rows, slice_width, group)
+        b.set_launch(0, thread_num_in_block=threads)
+        b.compile().upload(gpu)
+        print("case: row ownership", rows, cols, len(r), slice_width, group, threads, sort, runs, flush=True)
+        assert not b.clears_y() and "cur_group" in b.kernel_source()
+        assert_y(b.spmv(x), y_ref, mag, npd, "tile template, row ownership")
+        assert_y(b.spmv_device(x), y_ref, mag, npd, "tile template, row ownership, y = NaN before the call")
+        b.close()
+
+
 @pytest.mark.parametrize("position", [K.END_PADDING, K.TOP_PADDING], ids=["end", "top"])
 @pytest.mark.parametrize("skel,kw", [("S5", {}), ("S1", {"m": 64}), ("T1", {"slice": 1024, "group": 512, "b": 2048})],
                          ids=["S5", "S1", "T1"])
