@@ -31,7 +31,15 @@ static const uint64_t kCuNum = 256;
 static const uint64_t kUnit = 256;          // elements of one wavefront step of the first pass (64 lanes x 4)
 static const unsigned kBatch = 2;           // wavefront steps whose loads are in flight together
 static const uint64_t kBand = 4096;         // rows of y whose rows of the strip are summed and stored together
-static const unsigned kYPrefetch = 4;        // rows of a lane whose place in y is read ahead in the second pass
+// Rows of a lane whose place in y is read ahead in the second pass: as many as a lane has in the summing group of
+// an average row (`typical_group_rows`: the groups' sizes averaged over the rows), between 4 and 8.  Rows beyond them read their place between the stores of the rows before, one round trip
+// each (C5, 5-16 rows per lane: second pass 43.6 us with 4, 40.2 with 8, 44.3 with 12, 45.9 with 16 -- the loads
+// are issued for every lane whether its group has that many rows or not, and skipping them by a test on the
+// group's size cost more than it saved, 45.0; C3, 2.6 rows per lane: 15.7 us with 2 or 4, 16.1 with 9).
+static unsigned y_prefetch(const Template &t) {
+  const uint64_t per_lane = (t.sc("typical_group_rows") + t.finish_thread_num - 1) / std::max<uint64_t>(1, t.finish_thread_num);
+  return (unsigned)std::min<uint64_t>(8, std::max<uint64_t>(4, per_lane));
+}
 static const uint64_t kShortRow = 4;        // longest row that is taken band by band
 
 bool is_supported(const Matrix &m, uint64_t sub) {
@@ -241,6 +249,11 @@ std::unique_ptr<Template> init(const Matrix &m, uint64_t sub) {
   AS_CHECK(max_slots <= 65536 && max_slots * vs <= kLdsBytes, "a row group does not fit its LDS slots");
   t->scalar["max_slots"] = max_slots;
   t->scalar["sum_group_num"] = nsum;
+  {
+    uint64_t squares = 0;
+    for (uint64_t q = 0; q < nsum; q++) squares += (sum_first_row[q + 1] - sum_first_row[q]) * (sum_first_row[q + 1] - sum_first_row[q]);
+    t->scalar["typical_group_rows"] = squares / std::max<uint64_t>(1, sub_rows);
+  }
   const uint64_t product_len = slot.size();
   AS_CHECK(product_len < (1ull << 32), "sub-matrix too large for 32-bit element offsets");
   // first-pass padding goes to a spare slot behind the products
@@ -403,8 +416,8 @@ std::string kernel_source(const Template &t) {
   s += "    " + code_of_meta_read(t, "sum_group_width", "width", "grp");
   s += "    const unsigned int live = row_end - row0;\n";
   // the places in y of the lane's first rows are requested now and used after the sums
-  s += "    unsigned int y_place[" + std::to_string(kYPrefetch) + "];\n";
-  s += "    #pragma unroll\n    for (int k = 0; k < " + std::to_string(kYPrefetch) + "; k++)\n    {\n";
+  s += "    unsigned int y_place[" + std::to_string(y_prefetch(t)) + "];\n";
+  s += "    #pragma unroll\n    for (int k = 0; k < " + std::to_string(y_prefetch(t)) + "; k++)\n    {\n";
   s += "      const unsigned int sub_row = row0 + min(threadIdx.x + k * " + FB + "u, live - 1u);\n";
   s += "      " + code_of_meta_read(t, "y_row_index", "y_place[k]", "sub_row");
   s += "    }\n";
@@ -428,14 +441,14 @@ std::string kernel_source(const Template &t) {
   s += "      }\n    }\n";
   s += "    __syncthreads();\n";
   const std::string y_off = (!t.global_sort_index && t.kernal_first_row_index != 0 ? " + " + std::to_string(t.kernal_first_row_index) + "u" : std::string());
-  s += "    #pragma unroll\n    for (int k = 0; k < " + std::to_string(kYPrefetch) + "; k++)\n    {\n";
+  s += "    #pragma unroll\n    for (int k = 0; k < " + std::to_string(y_prefetch(t)) + "; k++)\n    {\n";
   s += "      const unsigned int i = threadIdx.x + k * " + FB + "u;\n";
   s += "      if (i < live)\n      {\n";
   s += "        " + vt + " sum = 0;\n";
   s += "        for (unsigned int j = 0; j < width; j++) sum += slots[j * live + i];\n";
   s += "        device_y_arr[y_place[k]" + y_off + "] = sum;\n";
   s += "      }\n    }\n";
-  s += "    for (unsigned int i = threadIdx.x + " + std::to_string(kYPrefetch) + "u * " + FB + "u; i < live; i += " + FB + "u)\n    {\n";
+  s += "    for (unsigned int i = threadIdx.x + " + std::to_string(y_prefetch(t)) + "u * " + FB + "u; i < live; i += " + FB + "u)\n    {\n";
   s += "      " + vt + " sum = 0;\n";
   s += "      for (unsigned int j = 0; j < width; j++) sum += slots[j * live + i];\n";
   s += "      const unsigned int sub_row = row0 + i;\n";
