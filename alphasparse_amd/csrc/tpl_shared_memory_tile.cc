@@ -103,35 +103,74 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   uint64_t want = kCuNum * std::max<uint64_t>(1, kLdsBytes / ((S + R) * vs));
   want = std::max<uint64_t>(1, std::min<uint64_t>(want, (n + 16383) / 16384));
   std::vector<uint64_t> group_first_block{0};
-  // Row ownership (own_rows): the BLBs are taken row group by row group (inside a row group slice by slice) and
-  // a trip is a whole number of row groups, so that one workgroup holds every sum of its rows: the cells of a row
-  // group live in LDS across its slices, a cell is the row's place in the group, and at the end of the group the
-  // rows are STORED to y -- no atomics, no table of places, y needs no clear.  The price is one slice copy per
-  // (row group, slice) tile instead of one per trip and slice, and trips as coarse as row groups: the form is
-  // turned down (nullptr) where the copies would move more than a quarter of the element stream's bytes, where
-  // there are fewer trips than half the workgroups the device holds, or where the heaviest trip would take more
-  // than 1.2 times the average.  It fits matrices of many row groups that meet few
-  // slices each (banded matrices); strips of a few very long rows stay with the slice-by-slice order.
-  std::vector<uint64_t> blk_order(B), trip_first_row_group;
-  for (uint64_t b = 0; b < B; b++) blk_order[b] = b;
+  // Row ownership (own_rows): the elements are taken row group by row group and a trip is a whole number of row
+  // groups, so that one workgroup holds every sum of its rows: the cells of a row group live in LDS across its
+  // runs, a cell is the row's place in the group, and at the end of the group the rows are STORED to y -- no
+  // atomics, no table of places, y needs no clear.  The price is one copy of x into LDS per run of every row group
+  // instead of one per trip and slice, and trips as coarse as row groups: the form is turned down (nullptr) where
+  // the copies would move more than a quarter of the element stream's bytes, where there are fewer trips than half
+  // the workgroups the device holds, or where the heaviest trip would take more than 1.2 times the average.  It
+  // fits matrices of many row groups that meet few slices each (banded matrices); strips of a few very long rows
+  // stay with the slice-by-slice order.
+  // The runs of the element stream: elements [begin, end) of `order` (row ownership) or of the format's own order,
+  // the first column of the stretch of x the run reads, and its row group.
+  struct Run { uint64_t begin, end, col0, rg; };
+  std::vector<Run> runs;
+  std::vector<uint64_t> trip_first_run, trip_first_row_group;
+  std::vector<uint32_t> order;  // row ownership: element numbers of the format in the order of the stream
   if (own_rows) {
     if (sub_block_is_col_restricted(m, sub)) return nullptr;  // another sub-matrix adds to the same rows
+    AS_CHECK(n < (1ull << 32), "sub-matrix too large for 32-bit element offsets");
+    std::vector<uint64_t> blk_order(B);
+    for (uint64_t b = 0; b < B; b++) blk_order[b] = b;
     std::stable_sort(blk_order.begin(), blk_order.end(), [&](uint64_t x, uint64_t y) {
       return blk_rg[x] != blk_rg[y] ? blk_rg[x] < blk_rg[y] : blk_slice[x] < blk_slice[y];
     });
-    const uint64_t NG = (sub_rows + R - 1) / R;
-    std::vector<uint64_t> group_cost(NG, 0);
-    uint64_t tiles = 0, stream_cost = 0;
-    for (uint64_t i = 0; i < B; i++) {
-      const uint64_t b = blk_order[i];
-      group_cost[blk_rg[b]] += blk_cost[b];
-      stream_cost += blk_cost[b];
-      if (i == 0 || blk_rg[b] != blk_rg[blk_order[i - 1]] || blk_slice[b] != blk_slice[blk_order[i - 1]]) {
-        group_cost[blk_rg[b]] += slice_cost;
-        tiles++;
+    // A row group does not read x slice by slice of the format's grid but window by window: a window starts at the
+    // group's first column not yet covered (rounded down to a 16-byte boundary of x) and is col_slice columns wide.
+    // The rows of a banded matrix fit one window where they straddle two or three slices of the grid, and a window
+    // is one copy of x into LDS and one run.  Inside a window the elements go row by row.
+    const uint64_t NG = (sub_rows + R - 1) / R, align = 16 / vs;
+    std::vector<uint64_t> group_cost(NG, 0), group_first_own_run(NG + 1, 0);
+    uint64_t stream_cost = 0;
+    order.reserve(n);
+    std::vector<uint32_t> members, sorted;
+    std::vector<uint64_t> row_count(R + 1);
+    for (uint64_t i = 0; i < B;) {
+      const uint64_t g = blk_rg[blk_order[i]];
+      members.clear();
+      for (; i < B && blk_rg[blk_order[i]] == g; i++) {
+        const uint64_t b = blk_order[i];
+        group_cost[g] += blk_cost[b];
+        for (uint64_t k = bl.coo_begin[b]; k < bl.coo_begin[b + 1]; k++) members.push_back((uint32_t)k);
+      }
+      stream_cost += group_cost[g];
+      group_first_own_run[g] = runs.size();
+      for (uint64_t covered = 0;;) {
+        uint64_t lo = ~0ull;
+        for (uint32_t k : members)
+          if (col[k] >= covered && col[k] < lo) lo = col[k];
+        if (lo == ~0ull) break;
+        const uint64_t w0 = lo / align * align, w1 = w0 + S;
+        // the window's elements row by row (a stable counting sort: inside a row the order of the format stays)
+        std::fill(row_count.begin(), row_count.end(), 0);
+        uint64_t inside = 0;
+        for (uint32_t k : members)
+          if (col[k] >= covered && col[k] < w1) row_count[row[k] - g * R + 1]++, inside++;
+        for (uint64_t r = 0; r < R; r++) row_count[r + 1] += row_count[r];
+        sorted.resize(inside);
+        for (uint32_t k : members)
+          if (col[k] >= covered && col[k] < w1) sorted[row_count[row[k] - g * R]++] = k;
+        runs.push_back({order.size(), order.size() + inside, w0, g});
+        order.insert(order.end(), sorted.begin(), sorted.end());
+        group_cost[g] += slice_cost;
+        covered = w1;
       }
     }
-    if (tiles * slice_cost * 4 > stream_cost) return nullptr;
+    group_first_own_run[NG] = runs.size();
+    for (uint64_t g = NG; g-- > 0;)
+      if (group_cost[g] == 0) group_first_own_run[g] = group_first_own_run[g + 1];  // a row group without elements
+    if (runs.size() * slice_cost * 4 > stream_cost) return nullptr;
     uint64_t total = 0;
     for (uint64_t c : group_cost) total += c;
     // as many trips as workgroups fit, or the fewest more row groups per trip that make the trips even
@@ -152,14 +191,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     const uint64_t T = trip_first_row_group.size() - 1;
     // too few trips leave most CUs idle; uneven trips make the others wait for the heaviest
     if (T * 2 < want || heaviest * T * 10 > total * 12) return nullptr;
-    // BLB view of the trips, in the order of blk_order
-    group_first_block.clear();
-    uint64_t i = 0;
-    for (uint64_t tp = 0; tp < T; tp++) {
-      group_first_block.push_back(i);
-      while (i < B && blk_rg[blk_order[i]] < trip_first_row_group[tp + 1]) i++;
-    }
-    group_first_block.push_back(B);
+    for (uint64_t tp = 0; tp <= T; tp++) trip_first_run.push_back(group_first_own_run[trip_first_row_group[tp]]);
   } else {
   uint64_t total_cost = want * slice_cost;
   for (uint64_t b = 0; b < B; b++) {
@@ -182,8 +214,17 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     }
     group_first_block.push_back(B);
   }
+  // runs: maximal sequences of BLBs of one tile inside a trip
+  for (uint64_t g = 0; g + 1 < group_first_block.size(); g++) {
+    trip_first_run.push_back(runs.size());
+    for (uint64_t b = group_first_block[g], e; b < group_first_block[g + 1]; b = e) {
+      for (e = b + 1; e < group_first_block[g + 1] && blk_slice[e] == blk_slice[b] && blk_rg[e] == blk_rg[b];) e++;
+      runs.push_back({bl.coo_begin[b], bl.coo_begin[e], blk_slice[b] * S, blk_rg[b]});
+    }
   }
-  const uint64_t G = group_first_block.size() - 1;
+  trip_first_run.push_back(runs.size());
+  }
+  const uint64_t G = trip_first_run.size() - 1;
   t->scalar["group_num"] = G;
   t->own_rows = own_rows;
 
@@ -217,19 +258,13 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   lcol.reserve(n + G * kRunUnit);
   piece.reserve(n + G * kRunUnit);
   t->val_arr.reserve(n + G * kRunUnit);
+  auto elem = [&](uint64_t i) { return own_rows ? (uint64_t)order[i] : i; };
   for (uint64_t g = 0; g < G; g++) {
     group_first_run.push_back(run_slice.size());
-    uint64_t i = group_first_block[g], i_end = group_first_block[g + 1];
-    while (i < i_end) {
-      const uint64_t b = blk_order[i];
-      uint64_t e = i;
-      while (e < i_end && blk_slice[blk_order[e]] == blk_slice[b] && blk_rg[blk_order[e]] == blk_rg[b]) {
-        AS_CHECK(e == i || blk_order[e] == blk_order[e - 1] + 1, "the BLBs of a tile must follow each other");
-        e++;
-      }
-      const uint64_t col0 = blk_slice[b] * S, k0 = bl.coo_begin[b], k1 = bl.coo_begin[blk_order[e - 1] + 1];
+    for (uint64_t ri = trip_first_run[g]; ri < trip_first_run[g + 1]; ri++) {
+      const Run &run = runs[ri];
+      const uint64_t col0 = run.col0, row0 = run.rg * R;
       const uint64_t slice_len = std::min<uint64_t>(S, t->matrix_cols - t->kernal_first_col_index - col0);
-      const uint64_t row0 = blk_rg[b] * R;
       uint64_t pieces = 0, cur_piece = 0;
       // a zero-valued element on the current piece; in the column-run form its column continues the run where
       // that stays inside the slice, and otherwise opens a run at column 0
@@ -241,11 +276,11 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
         piece.push_back(cur_piece);
         t->val_arr.push_back(0.0);
       };
-      for (uint64_t k = k0; k < k1; k++) {
-        const uint64_t c = col[k] - col0;
-        const bool new_row = k == k0 || row[k] != row[k - 1];
+      for (uint64_t i = run.begin; i < run.end; i++) {
+        const uint64_t k = elem(i), c = col[k] - col0;
+        const bool first = i == run.begin, new_row = first || row[k] != row[elem(i - 1)];
         // row ownership: a row that does not follow its predecessor directly cannot share a lane with it
-        if (own_rows && new_row && k != k0 && row[k] != row[k - 1] + 1)
+        if (own_rows && new_row && !first && row[k] != row[elem(i - 1)] + 1)
           while (lcol.size() % kLaneElems) pad();
         if (column_runs) {
           if (lcol.size() % kLaneElems == 0) lane_runs = 0;
@@ -271,11 +306,10 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
         if (column_runs && lcol.size() % kLaneElems == 0) lane_runs = 0;
         pad();
       }
-      run_slice.push_back(blk_slice[b]);
-      run_row_group.push_back(blk_rg[b]);
+      run_slice.push_back(own_rows ? col0 : col0 / S);
+      run_row_group.push_back(run.rg);
       run_nz_begin.push_back(lcol.size() / kRunUnit);
       run_piece_begin.push_back(piece_target.size());
-      i = e;
     }
   }
   group_first_run.push_back(run_slice.size());
@@ -356,7 +390,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     t->arrays.push_back(std::move(a));
   };
   add("group_first_run", std::move(group_first_run), true);
-  add("run_slice", std::move(run_slice), true);
+  add(own_rows ? "run_col_begin" : "run_slice", std::move(run_slice), true);
   add("run_nz_begin", std::move(run_nz_begin), true);
   if (own_rows) {
     add("run_row_group", std::move(run_row_group), true);
@@ -374,18 +408,19 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   add("y_row_index", std::move(y_row), false);
   // the finish kernel's map (the main kernel has piece_target), or the map of the rows a workgroup owns
   t->find("y_row_index")->on_device = t->finish_tblock_num != 0 || (own_rows && t->global_sort_index);
-  add("group_first_block", std::move(group_first_block), false);  // BLB view of the trips, host only
-  t->find("group_first_block")->on_device = false;
   if (own_rows) {
     add("trip_first_row_group", std::move(trip_first_row_group), false);  // host only
     t->find("trip_first_row_group")->on_device = false;
+  } else {
+    add("group_first_block", std::move(group_first_block), false);  // BLB view of the trips, host only
+    t->find("group_first_block")->on_device = false;
   }
   tpl_shared_memory_tile::set_default_launch(*t);
   return t;
 }
 
 void try_all_compress(Template &t) {
-  for (const char *name : {"group_first_run", "run_slice", "run_nz_begin", "run_piece_begin", "run_row_group", "y_row_index"}) {
+  for (const char *name : {"group_first_run", "run_slice", "run_col_begin", "run_nz_begin", "run_piece_begin", "run_row_group", "y_row_index"}) {
     TArr *a = t.find(name);
     if (a && !a->c.active()) init_linear_compressor(a->a, a->c, true);
   }
@@ -445,7 +480,7 @@ std::string kernel_source(const Template &t) {
   // run == run_end is the write-back of the trip's last run
   s += "      unsigned int next_run = run + 1u, slice = 0xffffffffu, unit_begin = 0u, unit_end = 0u, piece_begin = 0u, piece_end = 0u, row_group = 0xffffffffu;\n";
   s += "      if (run < run_end)\n      {\n";
-  s += "        " + code_of_meta_read(t, "run_slice", "slice", "run");
+  s += "        " + code_of_meta_read(t, t.own_rows ? "run_col_begin" : "run_slice", "slice", "run");
   s += "        " + code_of_meta_read(t, "run_nz_begin", "unit_begin", "run");
   s += "        " + code_of_meta_read(t, "run_nz_begin", "unit_end", "next_run");
   if (t.own_rows) {
@@ -503,7 +538,8 @@ std::string kernel_source(const Template &t) {
   s += "      done_begin = piece_begin; done_end = piece_end;\n";
   }
   s += "      if (run < run_end && slice != cur_slice)\n      {\n";
-  s += "        const unsigned int col0 = slice * " + Ss + ";\n";
+  // under row ownership the table holds the first column of the run's stretch of x itself
+  s += "        const unsigned int col0 = slice" + (t.own_rows ? std::string() : " * " + Ss) + ";\n";
   s += "        const unsigned int slice_len = min(" + Ss + ", " + std::to_string(x_len) + "u - col0);\n";
   const std::string Ks2 = std::to_string(kBetweenRunsBatch);
   if (wide_copy) {

@@ -184,17 +184,21 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
     arr = {k: np.asarray(a[0]).astype(np.int64) for k, a in t["arrays"].items()}
     val = np.asarray(t["val_arr"][0] if isinstance(t["val_arr"], tuple) else t["val_arr"], np.float64)
     own_rows = "run_row_group" in arr   # row ownership: cells are rows of the run's row group, kept across its runs
-    gfr, rs, nzb, word, yrow, lcol = (arr["group_first_run"], arr["run_slice"], arr["run_nz_begin"], arr["lane_word"],
-                                      arr["y_row_index"], arr["col_index_arr"])
+    gfr, nzb, word, yrow, lcol = (arr["group_first_run"], arr["run_nz_begin"], arr["lane_word"],
+                                  arr["y_row_index"], arr["col_index_arr"])
+    # the first column of the stretch of x a run reads: a slice of the format's grid, or (row ownership) a window
+    # that starts at the row group's first column not yet covered, on a 16-byte boundary of x
+    rs = arr["run_col_begin"] if own_rows else arr["run_slice"] * slice_width
     if own_rows:
         rrg = arr["run_row_group"]
+        assert "run_slice" not in arr and (rs % chunk == 0).all()
         assert "piece_target" not in arr and "run_piece_begin" not in arr and len(rrg) == len(rs)
         # a trip is a whole number of row groups, a row group the runs of one trip that follow each other
         trip_of_run = np.repeat(np.arange(len(gfr) - 1), np.diff(gfr))
         for g in np.unique(rrg):
             runs = np.flatnonzero(rrg == g)
             assert (np.diff(runs) == 1).all() and len(set(trip_of_run[runs].tolist())) == 1
-            assert (np.diff(rs[runs]) > 0).all()                 # slice by slice inside the group
+            assert (np.diff(rs[runs]) >= slice_width).all()      # window by window inside the group, none overlapping
         assert (np.diff(rrg) >= 0).all()
     else:
         rpb, target = arr["run_piece_begin"], arr["piece_target"]
@@ -230,7 +234,8 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
         else:
             cells = np.zeros(rpb[run + 1] - rpb[run])
         touched = np.zeros(len(cells), np.int64)
-        prod = val[k0:k1] * x[rs[run] * slice_width + lcol[k0:k1]]
+        assert (rs[run] + lcol[k0:k1] < len(x)).all()            # padding included: the kernel reads x there
+        prod = val[k0:k1] * x[rs[run] + lcol[k0:k1]]
         for u in range(0, k1 - k0, 512):                         # one wavefront step
             w = word[(k0 + u) // 8:(k0 + u) // 8 + 64]
             first = w & 0x7fff
@@ -340,8 +345,8 @@ def test_tile_division_and_tile_template(slice_width, group, blb, sort):
                          ids=["plain", "sorted", "plain_runs", "sorted_runs"])
 def test_tile_template_under_row_ownership(vdt, chunk, sort, runs):
     """set_row_ownership on a banded matrix of dense 3 x 3 blocks (many row groups, two or three slices each): the
-    tiles row group by row group, cells = rows of the group kept across its slices, lanes closed where a row of the
-    group is missing from a slice, no piece tables, no scratch, no atomics into y -- and the same y when the arrays
+    elements row group by row group and inside a group window by window of x, cells = rows of the group kept across
+    its windows, lanes closed where a row of the group is missing from a window, no piece tables, no scratch, no atomics into y -- and the same y when the arrays
     are walked the way the kernel walks them, alone and on top of the column-run form.  Turned down where it does
     not fit: a few long rows (one row group for all CUs), a column band, another template."""
     from alphasparse_amd import skeletons as SK
@@ -364,6 +369,10 @@ def test_tile_template_under_row_ownership(vdt, chunk, sort, runs):
     assert ("col_run_mask" in t["arrays"]) == runs and "run_row_group" in t["arrays"]
     assert t["scalars"]["is_atom_add"] == 0 and not b.clears_y()
     assert b.get_launch(0)["thread_num_in_block"] == 256
+    if not sort:
+        # 100 rows and their band of +-180 columns fit one window of 500 columns, wherever the grid's slices fall:
+        # one run and one copy of x per row group (the tiles of the format are two or three per row group)
+        assert len(t["arrays"]["run_col_begin"][0]) == -(-rows // 100) < len(before["arrays"]["run_slice"][0])
     vv = np.float32(v).astype(np.float64) if vdt == K.FLOAT else v.astype(np.float64)
     yref = np.zeros(rows)
     np.add.at(yref, np.asarray(r, np.int64), vv * x[np.asarray(c, np.int64)])
