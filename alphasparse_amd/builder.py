@@ -39,6 +39,8 @@ def _bind(L):
     L.as_builder_set_row_ownership.argtypes = [vp, C.c_int64]
     L.as_builder_set_x.argtypes = [vp, vp]
     L.as_builder_set_serial_launch.argtypes = [vp, C.c_int]
+    L.as_builder_set_finish_carry.argtypes = [vp, C.c_int]
+    L.as_builder_finish_carrier.argtypes = [vp, C.c_uint64, C.POINTER(C.c_int64)]
     L.as_builder_time_sub_matrix.argtypes = [vp, C.c_int64, C.c_uint64, C.POINTER(C.c_float), C.POINTER(C.c_uint64),
                                              C.POINTER(C.c_uint64), C.POINTER(C.c_int)]
     L.as_builder_time_sub_matrix_pass.argtypes = [vp, C.c_int64, C.c_int, C.c_uint64, C.POINTER(C.c_float)]
@@ -256,6 +258,18 @@ class Builder:
     def set_serial_launch(self, serial=True):
         self._chk(self._L.as_builder_set_serial_launch(self._h, int(bool(serial))))
         return self
+
+    def set_finish_carry(self, on=True):
+        """With serial launch: let the first kernel of a product-bin strip do the work of the finish kernel of the
+        tile strip in front of it (default on)."""
+        self._chk(self._L.as_builder_set_finish_carry(self._h, int(bool(on))))
+        return self
+
+    def finish_carrier(self, sub):
+        """The sub-matrix whose first kernel carries the finish of `sub`, or -1."""
+        out = C.c_int64(-1)
+        self._chk(self._L.as_builder_finish_carrier(self._h, sub, C.byref(out)))
+        return out.value
 
     def time(self, reps, sync_each_launch=False):
         ms, gf = C.c_float(0), C.c_float(0)

@@ -268,6 +268,8 @@ int as_builder_time_sub_matrix_pass(as_builder *b, int64_t sub, int pass, uint64
   bd.only_pass = pass;
   float gf = 0;
   asx::time_spmv(bd, reps, false, *time_ms, gf);
+  // a first kernel that adds into a scratch vector its finish kernel leaves cleared: cleared here instead
+  if (pass == 1 && bd.subs[sub].tpl->scratch_starts_zero) asx::clear_scratch(bd, (uint64_t)sub);
   return 0;
   AS_API_END(-1)
 }
@@ -283,7 +285,26 @@ int as_kernel_cache_stats(uint64_t *entries, uint64_t *hits) {
 int as_builder_set_serial_launch(as_builder *b, int serial) {
   AS_API_BEGIN
   AS_CHECK(b && b->b, "null builder");
+  if (b->b->serial_launch != (serial != 0)) asx::invalidate_module(*b->b);  // which finish kernels are carried changes
   b->b->serial_launch = serial != 0;
+  return 0;
+  AS_API_END(-1)
+}
+
+int as_builder_set_finish_carry(as_builder *b, int on) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b, "null builder");
+  if (b->b->carry_finish != (on != 0)) asx::invalidate_module(*b->b);
+  b->b->carry_finish = on != 0;
+  return 0;
+  AS_API_END(-1)
+}
+
+int as_builder_finish_carrier(as_builder *b, uint64_t sub, int64_t *carrier) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b && carrier, "null argument");
+  AS_CHECK(sub < b->b->subs.size() && b->b->subs[sub].tpl, "sub-matrix has no template");
+  *carrier = asx::assign_finish_carriers(*b->b, sub);
   return 0;
   AS_API_END(-1)
 }

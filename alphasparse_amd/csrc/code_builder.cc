@@ -178,7 +178,29 @@ bool set_column_runs(Builder &b, uint64_t sub) {
   return true;
 }
 
+int64_t assign_finish_carriers(const Builder &b, uint64_t sub) {
+  int64_t carrier_of_sub = -1;
+  const SubKernel *before = nullptr;
+  for (auto &k : b.subs) {
+    if (!k.tpl) continue;
+    k.tpl->carried = nullptr;
+    k.tpl->carried_blocks = 0;
+    // the strip before leaves its rows in a scratch vector for a finish kernel, and this one starts with a kernel
+    // that does not touch y: the two are independent, and the rows of the strip before are this kernel's to move
+    if (b.serial_launch && b.carry_finish && before && before->tpl->type == SHARED_MEMORY_TILE_TEMPLATE &&
+        before->tpl->finish_tblock_num && before->tpl->scratch_bytes && k.tpl->type == SHARED_MEMORY_PRODUCT_BIN_TEMPLATE) {
+      const uint64_t rows = before->tpl->sc("sub_rows"), threads = std::max<uint64_t>(64, k.tpl->thread_num_in_block);
+      k.tpl->carried = before->tpl.get();
+      k.tpl->carried_blocks = std::min<uint64_t>(256, ((rows + threads - 1) / threads + 7) / 8 * 8);
+      if (before->tpl->sub == sub) carrier_of_sub = (int64_t)k.tpl->sub;
+    }
+    before = &k;
+  }
+  return carrier_of_sub;
+}
+
 std::string build_module_source(const Builder &b) {
+  assign_finish_carriers(b);
   std::string s = kernel_module_preamble();
   s += "extern \"C\" __global__ void as_zero_words(unsigned int *p, unsigned long long n)\n{\n"
        "  for (unsigned long long i = blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x; i < n;\n"
@@ -309,18 +331,27 @@ static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned 
   bool multi = active > 1 && !b.serial_launch;
   if (multi) HIPL(as_hip_event_record(b.start_ev, b.main_stream));
   uint64_t scratch_offset = 0;
-  for (auto &k : b.subs) {
+  const SubKernel *before = nullptr;  // the sub-matrix with a template in front of the current one
+  void *scratch_before = nullptr;
+  for (size_t idx = 0; idx < b.subs.size(); idx++) {
+    SubKernel &k = b.subs[idx];
     void *scratch_ptr = k.scratch.ptr;
     if (k.tpl && k.tpl->scratch_bytes && static_scratch) {
       scratch_ptr = static_scratch + scratch_offset;
       scratch_offset += (k.tpl->scratch_bytes + 255) / 256 * 256;
+    }
+    const SubKernel *guest = before;
+    void *guest_scratch = scratch_before;
+    if (k.tpl) {
+      before = &k;
+      scratch_before = scratch_ptr;
     }
     if (skipped(k)) continue;
     AS_CHECK(k.uploaded && k.fn, "a template was changed after upload: call upload again");
     // kernel arguments: passed metadata arrays, val, col, x, y, scratch -- a fixed-size list, nothing allocated
     void *ptrs[kMaxKernelArgs], *args[kMaxKernelArgs];
     size_t n = 0;
-    AS_CHECK(k.meta.size() + 5 <= kMaxKernelArgs, "too many kernel arguments");
+    AS_CHECK(k.meta.size() + 8 <= kMaxKernelArgs, "too many kernel arguments");
     for (auto &m : k.meta) ptrs[n++] = m.ptr;
     ptrs[n++] = k.val.ptr;
     ptrs[n++] = k.col.ptr;
@@ -328,12 +359,42 @@ static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned 
     ptrs[n++] = y_dev;
     if (k.tpl->scratch_bytes) ptrs[n++] = scratch_ptr;
     for (size_t i = 0; i < n; i++) args[i] = &ptrs[i];
+    // A first kernel that carries the finish of the strip before it takes that strip's scratch vector, its places
+    // in y and its number of rows behind its own arguments -- 0 rows when this strip is launched alone.
+    size_t n_first = n;
+    unsigned int carried_rows = 0;
+    if (k.tpl->carried) {
+      AS_CHECK(guest && guest->tpl.get() == k.tpl->carried && guest->uploaded, "a template was changed after upload: call upload again");
+      ptrs[n_first] = guest_scratch;
+      args[n_first] = &ptrs[n_first];
+      n_first++;
+      if (carried_place_is_passed(*guest->tpl)) {
+        size_t at = 0;
+        for (auto &a : guest->tpl->arrays) {
+          if (a.name == "y_row_index") break;
+          at += a.passed();
+        }
+        ptrs[n_first] = guest->meta[at].ptr;
+        args[n_first] = &ptrs[n_first];
+        n_first++;
+      }
+      if (b.only_sub < 0) carried_rows = (unsigned int)guest->tpl->sc("sub_rows");
+      args[n_first++] = &carried_rows;
+    }
+    // ... and the strip before it then launches no finish kernel of its own
+    bool finish_is_carried = false;
+    if (b.only_sub < 0)
+      for (size_t j = idx + 1; j < b.subs.size(); j++)
+        if (b.subs[j].tpl) {
+          finish_is_carried = b.subs[j].tpl->carried == k.tpl.get();
+          break;
+        }
     void *s = multi ? k.stream : b.main_stream;
     if (multi) HIPL(as_hip_stream_wait_event(s, b.start_ev));
     if (b.only_pass != 2)
-      HIPL(as_hip_launch(k.fn, (unsigned)k.tpl->tblock_num, (unsigned)k.tpl->thread_num_in_block,
+      HIPL(as_hip_launch(k.fn, (unsigned)(k.tpl->tblock_num + k.tpl->carried_blocks), (unsigned)k.tpl->thread_num_in_block,
                          (unsigned)k.tpl->dynamic_lds_bytes, s, args));
-    if (k.tpl->finish_tblock_num && b.only_pass != 1) {
+    if (k.tpl->finish_tblock_num && b.only_pass != 1 && !finish_is_carried) {
       AS_CHECK(k.finish_fn, "a template was changed after upload: call upload again");
       HIPL(as_hip_launch(k.finish_fn, (unsigned)k.tpl->finish_tblock_num, (unsigned)k.tpl->finish_thread_num,
                          (unsigned)k.tpl->finish_lds_bytes, s, args));
@@ -353,6 +414,14 @@ static void zero_words(Builder &b, void *p, unsigned long long words) {
 
 static void zero_y(Builder &b, void *y_dev) {
   zero_words(b, y_dev, (unsigned long long)b.rows * dtype_size(b.val_dtype) / 4);
+}
+
+void clear_scratch(Builder &b, uint64_t sub) {
+  AS_CHECK(b.device_ready && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template on the device");
+  SubKernel &k = b.subs[sub];
+  if (!k.tpl->scratch_bytes || !k.scratch.ptr) return;
+  zero_words(b, k.scratch.ptr, (k.tpl->scratch_bytes + 3) / 4);
+  HIPL(as_hip_stream_sync(b.main_stream));
 }
 
 bool y_needs_clear(const Builder &b) {

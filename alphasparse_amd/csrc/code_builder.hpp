@@ -43,6 +43,10 @@ struct Builder {
   // false: every sub-matrix kernel runs on its own stream, all at once; true: one after the other on
   // the caller's stream (kernels that each fill the machine only get in each other's way)
   bool serial_launch = false;
+  // With serial_launch: the finish kernel of a tile-template strip is not launched where the strip after it has a
+  // product-bin template; the first workgroups of that template's first kernel do its work instead (see
+  // assign_finish_carriers).  false: every template launches its own kernels.
+  bool carry_finish = true;
   // >= 0: launches and timing cover the kernels of this sub-matrix only (per-kernel measurement)
   int64_t only_sub = -1;
   int only_pass = 0;  // with only_sub: 1 = the first kernel alone, 2 = the finish kernel alone, 0 = both
@@ -75,6 +79,12 @@ void load_and_upload(Builder &b, int device);     // module load + arrays to HBM
 // no kernel (rows removed by remove_empty_rows, a sub-matrix without template) or holds no element.  Graphs whose
 // kernels store every row exactly once (ELL / SELL strips, the two-kernel LDS templates) skip the clear.
 bool y_needs_clear(const Builder &b);
+// Zeroes the scratch array of one sub-matrix's kernels (after its first kernel ran without its finish kernel).
+void clear_scratch(Builder &b, uint64_t sub);
+// Decides which finish kernels are carried by the strip launched next (Template::carried of the carrying
+// template), from the templates, serial_launch and carry_finish; build_module_source calls it.  Returns the
+// sub-matrix whose first kernel carries the finish of `sub`, or -1.
+int64_t assign_finish_carriers(const Builder &b, uint64_t sub = ~0ull);
 // y = A x on device buffers already holding x; y is cleared first where y_needs_clear says so.
 void launch_spmv(Builder &b, const void *x_dev, void *y_dev);
 // The same SpMV for callers that must not allocate device memory: nothing is compiled, loaded or allocated

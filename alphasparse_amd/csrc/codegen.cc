@@ -25,10 +25,10 @@ __device__ __forceinline__ void as_atomic_add(double *p, double v) { unsafeAtomi
 // its own L2.  A kernel whose neighbouring blocks read neighbouring pieces of x takes its block number from
 // here instead of blockIdx.x: every XCD then works on a contiguous eighth of the blocks, and a line of x
 // that two neighbouring blocks need is fetched into one L2, not two.  A permutation of [0, gridDim.x).
-__device__ __forceinline__ unsigned int as_xcd_block_index() {
-  const unsigned int n = gridDim.x, b = blockIdx.x;
+__device__ __forceinline__ unsigned int as_xcd_block_index(unsigned int b, unsigned int n) {
   return b < (n & ~7u) ? (b & 7u) * (n >> 3) + (b >> 3) : b;
 }
+__device__ __forceinline__ unsigned int as_xcd_block_index() { return as_xcd_block_index(blockIdx.x, gridDim.x); }
 
 // One DPP move of a 32- or 64-bit value; lanes without a valid source read 0.
 template <int CTRL, int ROW_MASK, int BANK_MASK> __device__ __forceinline__ float as_dpp(float v) {
@@ -104,6 +104,44 @@ std::string kernel_signature(const Template &t) {
   s += "const " + vt + " *__restrict__ val_arr, const " + std::string(dtype_c_name(t.col_index_arr.dt)) +
        " *__restrict__ col_index_arr, const " + vt + " *__restrict__ device_x_arr, " + vt + " *__restrict__ device_y_arr";
   if (t.scratch_bytes) s += ", unsigned int *__restrict__ scratch_arr";
+  return s;
+}
+
+bool carried_place_is_passed(const Template &guest) { return guest.arr("y_row_index").passed(); }
+
+std::string carried_finish_signature(const Template &host) {
+  if (!host.carried) return std::string();
+  const Template &g = *host.carried;
+  std::string s = ", " + value_type_name(g) + " *__restrict__ carried_sum";
+  if (carried_place_is_passed(g))
+    s += std::string(", const ") + dtype_c_name(g.arr("y_row_index").a.dt) + " *__restrict__ carried_place";
+  return s + ", unsigned int carried_rows";
+}
+
+std::string carried_finish_prologue(const Template &host, uint64_t threads) {
+  if (!host.carried) return "  const unsigned int as_block = blockIdx.x, as_grid = gridDim.x;\n";
+  const Template &g = *host.carried;
+  const TArr &place = g.arr("y_row_index");
+  const std::string GB = std::to_string(host.carried_blocks) + "u", B = std::to_string(threads) + "u";
+  // The rows of the strip before this one wait in its scratch vector for their places in y: a few workgroups of
+  // this kernel move them there (and leave the vector cleared) while the others start on their own work, instead
+  // of a kernel of its own between the two strips -- a launch and a chain of two memory round trips that nothing
+  // overlapped.  A whole number of eights of workgroups, so that the others keep their XCDs.
+  std::string s;
+  s += "  if (blockIdx.x < " + GB + ")\n  {\n";
+  s += "    for (unsigned int sub_row = blockIdx.x * " + B + " + threadIdx.x; sub_row < carried_rows; sub_row += " + GB + " * " + B + ")\n    {\n";
+  s += "      const " + value_type_name(g) + " sum = carried_sum[sub_row];\n";
+  s += "      carried_sum[sub_row] = 0;\n";
+  s += "      unsigned int global_row_index;\n";
+  if (place.c.active()) {
+    s += "      " + code_of_arr_read(place.c, "global_row_index", "sub_row");
+    if (place.c.type != BRANCH_COMPRESS) s += ";\n";
+  } else {
+    s += "      global_row_index = carried_place[sub_row];\n";
+  }
+  s += "      as_stnt(device_y_arr + global_row_index, sum);\n";
+  s += "    }\n    return;\n  }\n";
+  s += "  const unsigned int as_block = blockIdx.x - " + GB + ", as_grid = gridDim.x - " + GB + ";\n";
   return s;
 }
 

@@ -835,6 +835,8 @@ bool search_dense_strategy(Ctx &c, const CooInput &in, std::vector<StrategyNode>
     // kernels that each fill the machine can be faster one after the other than on concurrent streams
     float ms = 0, gf = 0;
     bg.builder->serial_launch = true;
+    invalidate_module(*bg.builder);  // one after the other a finish kernel may be carried by the next strip's kernel
+    verify_candidate(c, *bg.builder, *bg.matrix, -1);
     time_builder(c, *bg.builder, ms, gf);
     c.log("combined graph: " + std::to_string(out.gflops) + " GFLOP/s on concurrent streams, " + std::to_string(gf) + " one after the other" + c.stamp());
     if (gf > out.gflops) { out.gflops = gf; out.time_ms = ms; out.serial_launch = true; }

@@ -84,6 +84,12 @@ struct Template {
   // slices and stores the rows to y at the end -- no atomics, no clear of y (no upstream counterpart; matrices of
   // many row groups that meet few slices each): see init_tile_template_variant
   bool own_rows = false;
+  // Carried finish (set by the builder when it writes the module, see assign_finish_carriers): the first
+  // `carried_blocks` workgroups of this template's first kernel do the work of the finish kernel of `carried`, the
+  // template of the row strip launched before this one, and leave; the other workgroups number themselves from 0.
+  // Not owned; nullptr = none.
+  const Template *carried = nullptr;
+  uint64_t carried_blocks = 0;
   // LDS the kernel asks for at launch (beyond its static __shared__ arrays)
   uint64_t dynamic_lds_bytes = 0;
   // Device scratch of the kernels (last argument `scratch_arr`): allocated and cleared once at upload; what
@@ -197,6 +203,14 @@ std::string kernel_module_preamble();
 // "const <type>* __restrict__ <name>, " for every passed metadata array, then
 // val/col/x/y.
 std::string kernel_signature(const Template &t);
+// A kernel that can carry another template's finish (Template::carried) appends carried_finish_signature to its
+// parameters and opens its body with carried_finish_prologue: the code of the carrying workgroups, then the
+// definitions of as_block / as_grid, the number of this workgroup among the kernel's own and how many those are.
+// `threads` = the kernel's workgroup size.  Extra launch arguments in order: the carried template's scratch
+// vector, its y_row_index array where that is passed, the number of its rows (0 = nothing to do this launch).
+std::string carried_finish_signature(const Template &host);
+std::string carried_finish_prologue(const Template &host, uint64_t threads);
+bool carried_place_is_passed(const Template &guest);
 // "<type> <var>;  <var> = name[idx] | closed form;" honouring compression.
 std::string code_of_meta_read(const Template &t, const std::string &arr, const std::string &var,
                               const std::string &idx);

@@ -350,7 +350,8 @@ std::string kernel_source(const Template &t) {
   std::string s;
   // ---- first pass: products -------------------------------------------------------------------
   s += "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(t.thread_num_in_block) + ") spmv_" + id + "(" +
-       kernel_signature(t) + ")\n{\n";
+       kernel_signature(t) + carried_finish_signature(t) + ")\n{\n";
+  s += carried_finish_prologue(t, t.thread_num_in_block);
   const std::string Cs = std::to_string(16 / dtype_size(t.val_dtype));
   s += "  typedef " + vt + " val16_t __attribute__((ext_vector_type(" + Cs + ")));\n";  // 16 bytes of values
   s += "  extern __shared__ __attribute__((aligned(16))) unsigned char as_dynamic_lds[];\n";
@@ -359,7 +360,7 @@ std::string kernel_source(const Template &t) {
   s += "  const unsigned int lane = threadIdx.x & 63u, wave_in_block = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);\n";
   s += "  const unsigned int stride = (" + B + " >> 6) * 256u;\n";
   s += "  const " + vt + " *x_sub = device_x_arr + " + std::to_string(t.kernal_first_col_index) + "u;\n";
-  s += "  for (unsigned int grp = as_xcd_block_index(); grp < " + std::to_string(G) + "u; grp += gridDim.x)\n  {\n";
+  s += "  for (unsigned int grp = as_xcd_block_index(as_block, as_grid); grp < " + std::to_string(G) + "u; grp += as_grid)\n  {\n";
   s += "    unsigned int next_grp = grp + 1u, slice, unit_begin, unit_end;\n";
   s += "    " + code_of_meta_read(t, "group_slice", "slice", "grp");
   s += "    " + code_of_meta_read(t, "group_first_unit", "unit_begin", "grp");

@@ -286,6 +286,14 @@ int64_t as_builder_static_scratch_need(as_builder *b);
 /* 0 (default): the kernels of the sub-matrices run concurrently, one stream each (code_builder.cc:1517-1518);
  * 1: one after the other on the caller's stream.  No counterpart in the reference. */
 int as_builder_set_serial_launch(as_builder *b, int serial);
+/* With serial launch: the finish kernel of a tile-template strip (the move of its row sums from the scratch vector
+ * to their places in y) is not launched where the strip after it has the product-bin template; the first
+ * workgroups of that template's first kernel, which does not touch y, do the move instead.  1 (default): on;
+ * 0: every template launches its own kernels.  Measurements of one sub-matrix alone always use its own kernels.
+ * as_builder_finish_carrier: the sub-matrix whose first kernel carries the finish of `sub` under the builder's
+ * current templates and settings, or -1.  No counterpart in the reference. */
+int as_builder_set_finish_carry(as_builder *b, int on);
+int as_builder_finish_carrier(as_builder *b, uint64_t sub, int64_t *carrier);
 /* `reps` back-to-back launches of the kernels of one sub-matrix only, timed with events on the launch stream;
  * also returns what that kernel's roofline figure is computed from: the bytes of its format arrays (padded
  * col + val + passed metadata), the rows of its strip and whether it accumulates y atomically.  No

@@ -552,6 +552,59 @@ def test_full_size_tile_and_product_bin_graphs(gpu, make, capsys):
     b.close()
 
 
+@pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
+def test_finish_of_a_tile_strip_carried_by_the_next_strips_kernel(gpu, vdt):
+    """Coarse sort, a tile strip (row sums through a scratch vector and a finish kernel) in front of a product-bin
+    strip, kernels one after the other: the finish kernel is not launched, the first workgroups of the product-bin
+    template's first kernel move the rows to y.  y against the oracle with the hand-over on and off, on y = NaN, call
+    after call (the scratch vector is left cleared), after measurements of one strip alone (which use the strip's
+    own kernels), and on concurrent streams (no hand-over)."""
+    rows, cols, r, c, v, x = S.power_law(30000, max_len=4000, mean_len=12.0, seed=11)
+    npd = NP[vdt]
+    v, x = v.astype(npd), x.astype(npd)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+    m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (16, 16, 2, 0))
+    m.execute_strategy(K.COMPRESS_NONE)
+    assert m.info()["n_sub"] == 2
+    b = A.Builder(m)
+    b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=1024, group=512, b=2048)[0])
+    b.set_template(1, SK.apply_skeleton(m, 1, "T2", slice=1024, group=4096, b=2048)[0])
+    y_ref, mag = oracle_y(rows, r, c, v, x)
+    z = np.random.default_rng(2).uniform(-1, 1, cols).astype(npd)
+    z_ref, z_mag = oracle_y(rows, r, c, v, z)
+    assert b.finish_carrier(0) == -1                             # concurrent streams: every strip its own kernels
+    b.set_serial_launch(True)
+    assert b.finish_carrier(0) == 1 and b.finish_carrier(1) == -1
+    for threads in (256, 1024):
+        b.set_launch(1, thread_num_in_block=threads)
+        b.compile().upload(gpu)
+        src = b.kernel_source()
+        assert "carried_sum" in src and "spmv_0_finish" in src and not b.clears_y()
+        print("case: carried finish, %d threads" % threads, flush=True)
+        assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, y = NaN before the call")
+        assert_y(b.spmv_device(z), z_ref, z_mag, npd, "carried finish, second call with another x")
+        assert_y(b.spmv_device(x, no_alloc=True), y_ref, mag, npd, "carried finish, static scratch")
+        # one strip alone: its own kernels (the tile strip its finish kernel, the product-bin kernel nothing to carry)
+        for sub in (0, 1):
+            assert b.time_sub_matrix(sub, 3)[0] > 0
+        assert b.time_sub_matrix_pass(1, 1, 3) > 0 and b.time_sub_matrix_pass(0, 1, 3) > 0 and b.time_sub_matrix_pass(0, 2, 3) > 0
+        assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, after the per-strip measurements")
+        ms, gf = b.time(5)
+        assert ms > 0
+        assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, after the timing loop")
+    b.set_finish_carry(False)
+    assert b.finish_carrier(0) == -1
+    b.compile().upload(gpu)
+    assert "carried_sum" not in b.kernel_source()
+    assert_y(b.spmv_device(x), y_ref, mag, npd, "finish kernel of its own")
+    b.set_finish_carry(True).set_serial_launch(False)
+    b.compile().upload(gpu)
+    assert "carried_sum" not in b.kernel_source()
+    assert_y(b.spmv_device(x), y_ref, mag, npd, "concurrent streams")
+    b.close()
+
+
 def test_missing_library_is_an_error_not_a_fallback():
     """The product has no CPU execution path: without the HIP library nothing runs."""
     import importlib
