@@ -57,6 +57,10 @@ PROFILE_OF = {"C2": "profiles/spmv_ell_c2_laplacian_hbm_traffic.txt", "C3": "pro
 # --copy-calibration).  Keyed by the first 16 hex digits of the SHA-256 of the generated module source: a graph
 # whose kernels changed in any way since it was profiled reports null and names the profile instead.
 MEASURED_TRAFFIC = {
+    "ff84531ca565a608": 117580800,    # C2, ELL kernel in diagonal form (pin S5,256,1,dia)
+    "e9afcd580f447551": 197734396,    # C3, tile kernel of the long strip + its finish (pin sort+div64|T1@1024|T2:slice=8192,group=65536@512)
+    "3b570d6d4c746c50": 803162829,    # C4, tile kernel, column runs under row ownership (pin |T1:slice=16384,group=4096@1024,runs,own)
+    "b9791554820cbb6f": 688027956,    # C5, product-bin kernel, both passes (pin sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256)
 }
 
 
