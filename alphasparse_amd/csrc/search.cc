@@ -630,8 +630,9 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
   // the same tiles in two passes (products streamed to scratch, then summed in small groups of rows): for
   // rows too short to leave several elements per slice, where every x read of a row-wise kernel would
   // bring a cache line from HBM.  k0: slice width = 128 KB of x, a quarter or a 32nd of it (narrow slices:
-  // several first-pass workgroups per CU, but shorter runs of products); k1: row group height 8192 or
-  // 65536 (the area the products of one slice trip are written to).
+  // several first-pass workgroups per CU, but shorter runs of products); k1: row group height 65536 or
+  // 8192 (the area the products of one slice trip are written to; the tall one first, it has won on every
+  // matrix measured so far and a search that runs out of time should have seen it).
   auto S12 = [&]() {
     Skeleton s;
     s.name = "S12";
@@ -644,7 +645,7 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
     s.nodes = [slice](const long *k) {
       static const int shift[] = {0, 2, 5};
       return std::vector<StrategyNode>{make_strategy(COMPRESSED_TBLOCK_LEVEL_COL_DIV_ROW_GROUP_COL_SLICE_PARAM_STRATEGY,
-                                                     slice >> shift[k[0]], k[1] ? 65536 : 8192, 8192)};
+                                                     slice >> shift[k[0]], k[1] ? 8192 : 65536, 8192)};
     };
     return s;
   };
