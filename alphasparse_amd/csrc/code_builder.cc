@@ -157,12 +157,15 @@ bool set_column_runs(Builder &b, uint64_t sub) {
   AS_CHECK(b.matrix != nullptr && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template");
   Template &old = *b.subs[sub].tpl;
   if (old.type != SHARED_MEMORY_TILE_TEMPLATE || old.col_runs) return false;
+  // worth it when the element stream gets shorter: the padding that closes lanes must not eat the 7 bytes per
+  // lane that the columns save.  Counted first (one pass over the columns), so that a matrix of scattered columns,
+  // where every element is a run of its own, is turned down before the form is built.
+  const double vs = (double)dtype_size(old.val_dtype);
+  const double before = (double)old.val_arr.size() * (vs + 2.5);
+  if ((double)tile_column_run_stream_estimate(*b.matrix, sub) * (vs + 1.625) > 0.98 * before) return false;
   std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, true, old.own_rows);
   if (!t) return false;
-  // worth it when the element stream gets shorter: the padding that closes lanes must not eat the 7 bytes per
-  // lane that the columns save
-  const double vs = (double)dtype_size(old.val_dtype);
-  const double before = (double)old.val_arr.size() * (vs + 2.5), after = (double)t->val_arr.size() * (vs + 1.625);
+  const double after = (double)t->val_arr.size() * (vs + 1.625);
   if (after > 0.98 * before) return false;
   try_all_compress(*t);
   t->y_needs_clear = template_needs_cleared_y(*t, *b.matrix, sub);

@@ -877,23 +877,34 @@ void sep_tblock_level_row_group_col_slice(CompressedBlock &cb, uint64_t S, uint6
   const uint64_t rows = sub_rows(cb), cols = ci.max_col - ci.min_col + 1;
   const uint64_t nrg = (rows + R - 1) / R, nsl = (cols + S - 1) / S;
   const std::vector<uint64_t> &row = ri.index_arr.v, &col = ci.index_arr.v;
+  AS_CHECK(n < (1ull << 32) && nsl * nrg < (1ull << 32), "sub-matrix too large for 32-bit element numbers");
   std::vector<uint64_t> tile_begin(nsl * nrg + 1, 0);
+  std::vector<uint32_t> tile_of(n);
   for (uint64_t k = 0; k < n; k++) {
     AS_CHECK(row[k] < rows && col[k] < cols, "element outside the sub-matrix");
-    tile_begin[(col[k] / S) * nrg + row[k] / R + 1]++;
+    tile_of[k] = (uint32_t)((col[k] / S) * nrg + row[k] / R);
+    tile_begin[tile_of[k] + 1]++;
   }
   for (size_t t = 0; t + 1 < tile_begin.size(); t++) tile_begin[t + 1] += tile_begin[t];
-  std::vector<uint64_t> nrow(n), ncol(n);
-  auto nval = std::make_shared<ValVec>(n);
+  // A stable counting sort by tile.  The elements' new places are written into one array of 32-bit numbers first
+  // and each of the three arrays is then gathered through it on its own: a scatter of all three at once keeps
+  // three open pages per tile, more than the TLB holds once there are a few hundred tiles.
+  std::vector<uint32_t> from(n);
   {
     std::vector<uint64_t> next(tile_begin.begin(), tile_begin.end() - 1);
-    for (uint64_t k = 0; k < n; k++) {
-      uint64_t p = next[(col[k] / S) * nrg + row[k] / R]++;
-      nrow[p] = row[k];
-      ncol[p] = col[k];
-      (*nval)[p] = (*cb.val)[k];
-    }
+    for (uint64_t k = 0; k < n; k++) from[next[tile_of[k]]++] = (uint32_t)k;
   }
+  std::vector<uint32_t>().swap(tile_of);
+  std::vector<uint64_t> nrow(n), ncol(n);
+  auto nval = std::make_shared<ValVec>(n);
+  for (uint64_t p = 0; p < n; p++) nrow[p] = row[from[p]];
+  for (uint64_t p = 0; p < n; p++) ncol[p] = col[from[p]];
+  {
+    const ValVec &val = *cb.val;
+    ValVec &out = *nval;
+    for (uint64_t p = 0; p < n; p++) out[p] = val[from[p]];
+  }
+  std::vector<uint32_t>().swap(from);
   std::vector<uint64_t> fr, rn, cbg, sz;
   uint64_t max_rn = 0, max_sz = 0;
   for (size_t t = 0; t + 1 < tile_begin.size(); t++)
@@ -908,9 +919,19 @@ void sep_tblock_level_row_group_col_slice(CompressedBlock &cb, uint64_t S, uint6
     }
   cbg.push_back(n);
   const uint64_t B = fr.size();
-  auto nri = std::make_shared<Index>(ri), nci = std::make_shared<Index>(ci);
-  nri->index_arr.assign(std::move(nrow), ri.index_arr.dt);
-  nci->index_arr.assign(std::move(ncol), ci.index_arr.dt);
+  // copies of the two COO levels with the re-ordered arrays in place of the old ones (which are not copied first)
+  auto with_array = [](const Index &src, std::vector<uint64_t> arr) {
+    auto out = std::make_shared<Index>();
+    out->level = src.level; out->ctype = src.ctype; out->itype = src.itype;
+    out->block_num = src.block_num; out->length = src.length;
+    out->first_row = src.first_row; out->row_number = src.row_number;
+    out->coo_begin = src.coo_begin; out->coo_block_size = src.coo_block_size;
+    out->max_row = src.max_row; out->min_row = src.min_row; out->max_col = src.max_col; out->min_col = src.min_col;
+    out->index_arr.assign(std::move(arr), src.index_arr.dt);
+    out->index_arr.present = src.index_arr.present;
+    return out;
+  };
+  auto nri = with_array(ri, std::move(nrow)), nci = with_array(ci, std::move(ncol));
   cb.read_index[0] = nri;
   cb.read_index[1] = nci;
   cb.val = nval;

@@ -988,6 +988,9 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
     for (long low : {512, 128, 32})
       for (long rate : {4, 8, 16}) bands.push_back({low, 2048, rate});
     std::vector<std::vector<uint64_t>> seen;
+    // A row division is a step of this level's search, and like the levels below it ends after steps in a row
+    // that bring nothing (three here: a step costs seconds on a large matrix, not milliseconds).
+    int struggle = 0;
     for (size_t bi = 0; bi < bands.size() && now_s() < T; bi++) {
       StrategyNode div = make_strategy(DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY, bands[bi][0], bands[bi][1], bands[bi][2], 0);
       std::vector<uint64_t> cut = strips_of(sorted_len, bands[bi][0], bands[bi][1], bands[bi][2]);
@@ -997,7 +1000,13 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
       c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
       BestGraph g;
       double budget = (T - now_s()) / 2;
-      if (search_dense_strategy(c, in, {input, sort, div, compress}, budget, g) && g.gflops > best3.gflops) best3 = g;
+      if (search_dense_strategy(c, in, {input, sort, div, compress}, budget, g) && g.gflops > best3.gflops) {
+        best3 = g;
+        struggle = 0;
+      } else if (best3.gflops > 0 && ++struggle >= 3) {
+        c.log("three row divisions in a row without an improvement: strategy 3 ends" + c.stamp());
+        break;
+      }
     }
     if (best3.gflops > 0) consider(best3, "strategy3");
   }

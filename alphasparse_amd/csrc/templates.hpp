@@ -167,6 +167,9 @@ std::unique_ptr<Template> init_tile_template_with_column_runs(const Matrix &m, u
 // ownership is asked for and does not fit the sub-matrix: a column band of the matrix, slice copies that would
 // move more than a quarter of the element stream's bytes, or trips (whole row groups) too uneven to fill the device.
 std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows);
+// Elements the tile template's stream would hold in the column-run form (lane-closing padding included), counted in
+// one pass without building the template: what set_column_runs looks at before it builds anything.
+uint64_t tile_column_run_stream_estimate(const Matrix &m, uint64_t sub);
 // HIP source of `extern "C" __global__ void spmv_<sub>(...)`.
 std::string code_of_template_kernal(const Template &t);
 // Kernel arguments in order: names of the metadata arrays that are passed

@@ -64,6 +64,39 @@ bool is_supported(const Matrix &m, uint64_t sub) {
 }
 
 static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows);
+
+// Elements the stream of the column-run form would hold, lane-closing padding included (the padding of runs to whole
+// wavefront steps left out): one pass over the columns, nothing built.  A lane takes eight elements and at most
+// kLaneRuns runs of consecutive columns; tiles start on a new lane.
+uint64_t column_run_stream_estimate(const Matrix &m, uint64_t sub) {
+  const CompressedBlock &cb = *m.items[sub].cb;
+  const Index &bl = *cb.read_index[2];
+  const uint64_t S = cb.col_slice, R = cb.row_group;
+  const std::vector<uint64_t> &row = cb.read_index[0]->index_arr.v, &col = cb.read_index[1]->index_arr.v;
+  uint64_t total = 0, fill = 0, runs = 0, prev = 0;
+  for (uint64_t b = 0; b < bl.block_num; b++) {
+    const uint64_t k0 = bl.coo_begin[b], k1 = bl.coo_begin[b + 1];
+    if (b > 0 && (col[k0] / S != col[bl.coo_begin[b - 1]] / S || row[k0] / R != row[bl.coo_begin[b - 1]] / R) && fill) {
+      total += kLaneElems - fill;
+      fill = 0;
+    }
+    for (uint64_t k = k0; k < k1; k++) {
+      if (fill == 0) runs = 0;
+      if (fill == 0 || col[k] != prev + 1) {
+        if (runs >= kLaneRuns) {
+          total += kLaneElems - fill;
+          fill = 0;
+          runs = 0;
+        }
+        runs++;
+      }
+      prev = col[k];
+      total++;
+      fill = (fill + 1) % kLaneElems;
+    }
+  }
+  return total + (fill ? kLaneElems - fill : 0);
+}
 std::unique_ptr<Template> init(const Matrix &m, uint64_t sub) { return build(m, sub, false, false); }
 std::unique_ptr<Template> init_with_column_runs(const Matrix &m, uint64_t sub) { return build(m, sub, true, false); }
 // nullptr when row ownership does not fit the sub-matrix (see build)
@@ -121,6 +154,16 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   if (own_rows) {
     if (sub_block_is_col_restricted(m, sub)) return nullptr;  // another sub-matrix adds to the same rows
     AS_CHECK(n < (1ull << 32), "sub-matrix too large for 32-bit element offsets");
+    // the rules below, on what is known before anything is re-ordered: there are no more trips than row groups,
+    // and a window of x covers at most two slices of the grid, so a row group has at least half as many runs as tiles
+    {
+      uint64_t tiles = 0, stream = 0;
+      for (uint64_t b = 0; b < B; b++) {
+        tiles += b == 0 || blk_slice[b] != blk_slice[b - 1] || blk_rg[b] != blk_rg[b - 1];
+        stream += blk_cost[b];
+      }
+      if ((sub_rows + R - 1) / R * 2 < want || (tiles + 1) / 2 * slice_cost * 4 > stream) return nullptr;
+    }
     std::vector<uint64_t> blk_order(B);
     for (uint64_t b = 0; b < B; b++) blk_order[b] = b;
     std::stable_sort(blk_order.begin(), blk_order.end(), [&](uint64_t x, uint64_t y) {
