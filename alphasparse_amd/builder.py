@@ -37,6 +37,7 @@ def _bind(L):
     L.as_builder_set_diagonal_columns.argtypes = [vp, C.c_int64]
     L.as_builder_set_column_runs.argtypes = [vp, C.c_int64]
     L.as_builder_set_row_ownership.argtypes = [vp, C.c_int64]
+    L.as_builder_set_row_blocks.argtypes = [vp, C.c_int64, C.c_int]
     L.as_builder_set_x.argtypes = [vp, vp]
     L.as_builder_set_serial_launch.argtypes = [vp, C.c_int]
     L.as_builder_set_finish_carry.argtypes = [vp, C.c_int]
@@ -133,6 +134,11 @@ class Builder:
         atomics); True when applied (upload again), False when the template is another one or the form does not
         fit the sub-matrix."""
         return bool(self._chk(self._L.as_builder_set_row_ownership(self._h, sub)))
+
+    def set_row_blocks(self, sub, rows_per_block):
+        """Tile template under row ownership: blocks of 2-4 consecutive rows that hold the same columns stored as
+        one piece; True when applied (upload again), False when the rows do not come in such blocks."""
+        return bool(self._chk(self._L.as_builder_set_row_blocks(self._h, sub, rows_per_block)))
 
     def get_launch(self, sub):
         out = (C.c_long * 4)()

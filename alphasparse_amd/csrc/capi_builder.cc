@@ -101,6 +101,13 @@ int as_builder_set_row_ownership(as_builder *b, int64_t sub) {
   AS_API_END(-1)
 }
 
+int as_builder_set_row_blocks(as_builder *b, int64_t sub, int rows_per_block) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b && sub >= 0 && rows_per_block >= 2 && rows_per_block <= 4, "bad argument");
+  return asx::set_row_blocks(*b->b, (uint64_t)sub, (uint64_t)rows_per_block) ? 1 : 0;
+  AS_API_END(-1)
+}
+
 int as_builder_set_column_runs(as_builder *b, int64_t sub) {
   AS_API_BEGIN
   AS_CHECK(b && b->b && sub >= 0, "bad argument");

@@ -153,6 +153,27 @@ bool set_row_ownership(Builder &b, uint64_t sub) {
   return true;
 }
 
+bool set_row_blocks(Builder &b, uint64_t sub, uint64_t rows_per_block) {
+  AS_CHECK(b.matrix != nullptr && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template");
+  AS_CHECK(rows_per_block >= 2 && rows_per_block <= 4, "blocks of 2, 3 or 4 rows");
+  Template &old = *b.subs[sub].tpl;
+  if (old.type != SHARED_MEMORY_TILE_TEMPLATE || !old.own_rows || old.row_block != 1) return false;
+  std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, old.col_runs, true, rows_per_block);
+  if (!t) return false;
+  try_all_compress(*t);
+  t->y_needs_clear = template_needs_cleared_y(*t, *b.matrix, sub);
+  t->thread_num_in_block = old.thread_num_in_block;
+  set_default_launch(*t);
+  if (b.subs[sub].uploaded) {
+    as_hip_device_sync();
+    free_sub_arrays(b.subs[sub]);
+    b.subs[sub].uploaded = false;
+  }
+  b.subs[sub].tpl = std::move(t);
+  invalidate(b);
+  return true;
+}
+
 bool set_column_runs(Builder &b, uint64_t sub) {
   AS_CHECK(b.matrix != nullptr && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template");
   Template &old = *b.subs[sub].tpl;
@@ -163,7 +184,7 @@ bool set_column_runs(Builder &b, uint64_t sub) {
   const double vs = (double)dtype_size(old.val_dtype);
   const double before = (double)old.val_arr.size() * (vs + 2.5);
   if ((double)tile_column_run_stream_estimate(*b.matrix, sub) * (vs + 1.625) > 0.98 * before) return false;
-  std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, true, old.own_rows);
+  std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, true, old.own_rows, old.row_block);
   if (!t) return false;
   const double after = (double)t->val_arr.size() * (vs + 1.625);
   if (after > 0.98 * before) return false;

@@ -69,6 +69,10 @@ bool set_column_runs(Builder &b, uint64_t sub);
 // is kept when it is in place); false (template unchanged) when the sub-matrix has another template, the form
 // is in place already or it does not fit the sub-matrix.  The launch setting is kept.
 bool set_row_ownership(Builder &b, uint64_t sub);
+// Tile template under row ownership: blocks of `rows_per_block` (2-4) consecutive rows that hold the same columns
+// stored as one piece (one set of columns and lane words for the block).  false where the rows do not come in
+// such blocks, the row group's height is not a multiple of the block, or the form is in place.
+bool set_row_blocks(Builder &b, uint64_t sub, uint64_t rows_per_block);
 // Whole module: preamble + every spmv_<sub> (code_of_kernal_define, build_main_file's kernel part)
 std::string build_module_source(const Builder &b);
 void compile_builder(Builder &b);                 // hipRTC, no GPU needed (compile_spmv_code, executor.cc:61)

@@ -35,6 +35,24 @@ MatrixInfo get_sub_matrix_info_from_compressed_matrix_block(const Matrix &m, uin
   i.max_row_nnz = *std::max_element(i.row_nnz.begin(), i.row_nnz.end());
   i.min_row_nnz = *std::min_element(i.row_nnz.begin(), i.row_nnz.end());
   i.avg_row_nnz = i.nnz / i.row_num;
+  // blocks of rows with the same columns, judged from the first 48 rows (elements are still row by row here)
+  if (m.items[sub].cb->read_index.size() == 2) {
+    const std::vector<uint64_t> &col = m.items[sub].cb->read_index[1]->index_arr.v;
+    std::vector<uint64_t> start{0};
+    for (uint64_t r = 0; r < std::min<uint64_t>(i.row_num, 48); r++) start.push_back(start.back() + i.row_nnz[r]);
+    const uint64_t rows = start.size() - 1;
+    for (uint64_t h : {4, 3, 2}) {
+      if (i.row_num % h != 0 || rows < 2 * h) continue;
+      bool same = true;
+      for (uint64_t blk = 0; same && blk < rows / h; blk++)
+        for (uint64_t q = 1; same && q < h; q++) {
+          const uint64_t a = start[blk * h], b = start[blk * h + q], len = start[blk * h + 1] - a;
+          same = start[blk * h + q + 1] - b == len;
+          for (uint64_t e = 0; same && e < len; e++) same = col[a + e] == col[b + e];
+        }
+      if (same) { i.row_block = h; break; }
+    }
+  }
   return i;
 }
 
@@ -104,6 +122,7 @@ std::string convert_template_node_to_string(const TemplateNode &n) {
     if (n.col_relative == 2) s += "col_index_diagonal:1\n";
     if (n.col_relative == 3) s += "col_index_runs:1\n";
     if (n.own_rows == 1) s += "y_rows_owned:1\n";
+    if (n.row_block > 1) s += "row_block:" + std::to_string(n.row_block) + "\n";
     // upstream closes every kernel node with one more "}" than it opened (exe_graph.cc:3547); kept,
     // since readers of test.log are written against that text
     return s + "}\n}\n";
@@ -429,6 +448,24 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
                 " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
                 " row ownership -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
           if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+          // and, where the rows come in blocks that hold the same columns, with a block of rows as one piece
+          const uint64_t height = best.own_rows == 1 ? tile_row_block_guess(m, sub) : 1;
+          if (height > 1 && set_row_blocks(*b, sub, height)) {
+            load_and_upload(*b, c.opt.device);
+            if (as_hip_h2d(b->x.ptr, c.probe_x.data(), b->x.bytes) != 0) throw Error(as_hip_last_error());
+            n.row_block = (long)height;
+            n.tblock_num = 0;
+            set_launch(*b->subs[sub].tpl, n);
+            invalidate_module(*b);
+            verify_candidate(c, *b, m, (int64_t)sub);
+            time_builder(c, *b, ms, gf);
+            c.res.candidates++;
+            n.tblock_num = (long)b->subs[sub].tpl->tblock_num;
+            c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
+                  " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
+                  " row blocks of " + std::to_string(height) + " -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
+            if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+          }
         }
       } catch (const std::exception &e) {
         c.res.failed_candidates++;
@@ -620,6 +657,9 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
     s.name = "S11";
     s.templates = {SHARED_MEMORY_TILE_TEMPLATE};
     long slice = (long)(131072 / (info.is_double ? 8 : 4)), group = slice / 4;
+    // rows that come in blocks of equal columns: row groups of whole blocks (halved groups too), so that the
+    // template can store a block of rows as one piece
+    if (info.row_block > 1) group = group / (2 * (long)info.row_block) * (2 * (long)info.row_block);
     s.knobs = [](ParamEnumerator &e, long *k) { e.add(&k[0], 0, 1, 1); };
     s.nodes = [slice, group](const long *k) {
       return std::vector<StrategyNode>{make_strategy(COMPRESSED_TBLOCK_LEVEL_COL_DIV_ROW_GROUP_COL_SLICE_PARAM_STRATEGY,
@@ -877,6 +917,8 @@ BuiltGraph build_from_graph(const CooInput &in, const BestGraph &g, unsigned wav
       AS_CHECK(set_column_runs(*r.builder, s), "the best graph's column runs cannot be rebuilt");
     if (g.subs[s].tpl.own_rows == 1)
       AS_CHECK(set_row_ownership(*r.builder, s), "the best graph's row ownership cannot be rebuilt");
+    if (g.subs[s].tpl.row_block > 1)
+      AS_CHECK(set_row_blocks(*r.builder, s, (uint64_t)g.subs[s].tpl.row_block), "the best graph's row blocks cannot be rebuilt");
     set_launch(*r.builder->subs[s].tpl, g.subs[s].tpl);
   }
   return r;

@@ -18,6 +18,9 @@ struct MatrixInfo {
   uint64_t nnz = 0, row_num = 0, col_num = 0, max_row_nnz = 0, min_row_nnz = 0, avg_row_nnz = 0;
   bool is_sorted = false;
   bool is_double = false;   // value type of the matrix
+  // 4, 3 or 2 where the first rows come in blocks of that many consecutive rows with the same columns (the dense
+  // blocks of a FEM matrix), else 1; only get_sub_matrix_info_from_compressed_matrix_block fills it
+  uint64_t row_block = 1;
 };
 MatrixInfo get_matrix_info(const Matrix &m);                                      // matrix_info.cc:22
 MatrixInfo get_sub_matrix_info_from_compressed_matrix_block(const Matrix &m, uint64_t sub);  // matrix_info.cc:140
@@ -56,6 +59,7 @@ struct TemplateNode {
   long col_relative = 0;
   // 1: tile template under row ownership (set_row_ownership)
   long own_rows = 0;
+  long row_block = 0;   // tile template: rows stored in blocks of this many (as_builder_set_row_blocks), 0 = not
 };
 std::string convert_template_node_to_string(const TemplateNode &n);   // exe_graph.cc:3317
 

@@ -84,6 +84,9 @@ struct Template {
   // slices and stores the rows to y at the end -- no atomics, no clear of y (no upstream counterpart; matrices of
   // many row groups that meet few slices each): see init_tile_template_variant
   bool own_rows = false;
+  // tile template under row ownership: rows come in blocks of this many consecutive rows with the same columns and
+  // are stored as such (1 = every row by itself): see init_tile_template_variant
+  uint64_t row_block = 1;
   // Carried finish (set by the builder when it writes the module, see assign_finish_carriers): the first
   // `carried_blocks` workgroups of this template's first kernel do the work of the finish kernel of `carried`, the
   // template of the row strip launched before this one, and leave; the other workgroups number themselves from 0.
@@ -166,7 +169,13 @@ std::unique_ptr<Template> init_tile_template_with_column_runs(const Matrix &m, u
 // SHARED_MEMORY_TILE_TEMPLATE in any combination of its two forms (column runs, row ownership); nullptr when row
 // ownership is asked for and does not fit the sub-matrix: a column band of the matrix, slice copies that would
 // move more than a quarter of the element stream's bytes, or trips (whole row groups) too uneven to fill the device.
-std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows);
+// row_block = b > 1 (only under row ownership): b consecutive rows that hold the same columns share their columns,
+// lane words and x reads; nullptr where some block of rows does not (or b does not divide the row group's height).
+std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows,
+                                                     uint64_t row_block = 1);
+// Height (4, 3, 2, else 1) of the blocks of rows with equal columns that a tile-divided sub-matrix seems to be made
+// of, judged from its first tile; what the search looks at before it tries init_tile_template_variant(.., row_block).
+uint64_t tile_row_block_guess(const Matrix &m, uint64_t sub);
 // Elements the tile template's stream would hold in the column-run form (lane-closing padding included), counted in
 // one pass without building the template: what set_column_runs looks at before it builds anything.
 uint64_t tile_column_run_stream_estimate(const Matrix &m, uint64_t sub);

@@ -164,15 +164,17 @@ std::unique_ptr<Template> init_tile_template_with_column_runs(const Matrix &m, u
   AS_CHECK(is_supported_by_template(SHARED_MEMORY_TILE_TEMPLATE, m, sub), "format is not supported by SHARED_MEMORY_TILE_TEMPLATE");
   return tpl_shared_memory_tile::init_with_column_runs(m, sub);
 }
-namespace tpl_shared_memory_tile { std::unique_ptr<Template> init_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows); }
+namespace tpl_shared_memory_tile { std::unique_ptr<Template> init_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows, uint64_t row_block); }
+namespace tpl_shared_memory_tile { uint64_t row_block_guess(const Matrix &m, uint64_t sub); }
+uint64_t tile_row_block_guess(const Matrix &m, uint64_t sub) { return tpl_shared_memory_tile::row_block_guess(m, sub); }
 namespace tpl_shared_memory_tile { uint64_t column_run_stream_estimate(const Matrix &m, uint64_t sub); }
 uint64_t tile_column_run_stream_estimate(const Matrix &m, uint64_t sub) {
   return tpl_shared_memory_tile::column_run_stream_estimate(m, sub);
 }
 
-std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows) {
+std::unique_ptr<Template> init_tile_template_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows, uint64_t row_block) {
   AS_CHECK(is_supported_by_template(SHARED_MEMORY_TILE_TEMPLATE, m, sub), "format is not supported by SHARED_MEMORY_TILE_TEMPLATE");
-  return tpl_shared_memory_tile::init_variant(m, sub, column_runs, own_rows);
+  return tpl_shared_memory_tile::init_variant(m, sub, column_runs, own_rows, row_block);
 }
 std::string code_of_template_kernal(const Template &t) { AS_DISPATCH(t.type, kernel_source(t)) }
 

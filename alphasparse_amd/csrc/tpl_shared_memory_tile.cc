@@ -63,7 +63,7 @@ bool is_supported(const Matrix &m, uint64_t sub) {
   return true;
 }
 
-static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows);
+static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows, uint64_t row_block = 1);
 
 // Elements the stream of the column-run form would hold, lane-closing padding included (the padding of runs to whole
 // wavefront steps left out): one pass over the columns, nothing built.  A lane takes eight elements and at most
@@ -100,16 +100,58 @@ uint64_t column_run_stream_estimate(const Matrix &m, uint64_t sub) {
 std::unique_ptr<Template> init(const Matrix &m, uint64_t sub) { return build(m, sub, false, false); }
 std::unique_ptr<Template> init_with_column_runs(const Matrix &m, uint64_t sub) { return build(m, sub, true, false); }
 // nullptr when row ownership does not fit the sub-matrix (see build)
-std::unique_ptr<Template> init_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows) {
-  return build(m, sub, column_runs, own_rows);
+std::unique_ptr<Template> init_variant(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows, uint64_t row_block) {
+  return build(m, sub, column_runs, own_rows, row_block);
 }
 
-static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows) {
+// The height of the blocks of rows the sub-matrix seems to be made of, from the rows of its first tile (up to 16
+// blocks): 4, 3 or 2 where that many consecutive rows (the first a multiple of the height, the height a divisor of
+// the row group's) hold the same columns block after block, else 1.  A guess that saves building a form that cannot
+// apply; the build itself checks every block.
+uint64_t row_block_guess(const Matrix &m, uint64_t sub) {
+  const CompressedBlock &cb = *m.items[sub].cb;
+  const Index &bl = *cb.read_index[2];
+  const uint64_t S = cb.col_slice, R = cb.row_group;
+  const std::vector<uint64_t> &row = cb.read_index[0]->index_arr.v, &col = cb.read_index[1]->index_arr.v;
+  uint64_t blbs = 1;
+  while (blbs < bl.block_num && col[bl.coo_begin[blbs]] / S == col[bl.coo_begin[0]] / S &&
+         row[bl.coo_begin[blbs]] / R == row[bl.coo_begin[0]] / R)
+    blbs++;
+  const uint64_t k0 = bl.coo_begin[0], k1 = bl.coo_begin[blbs];
+  std::vector<uint64_t> start;
+  for (uint64_t k = k0; k < k1 && start.size() <= 64; k++)
+    if (k == k0 || row[k] != row[k - 1]) start.push_back(k);
+  if (start.size() <= 64) start.push_back(k1);
+  const uint64_t rows = start.size() - 1;
+  for (uint64_t h : {4, 3, 2}) {
+    if (R % h != 0 || rows < h) continue;
+    bool same = true;
+    for (uint64_t blk = 0; same && blk < std::min<uint64_t>(rows / h, 16); blk++) {
+      const uint64_t f = blk * h, len = start[f + 1] - start[f];
+      same = row[start[f]] % h == 0;
+      for (uint64_t q = 1; same && q < h; q++) {
+        same = row[start[f + q]] == row[start[f]] + q && start[f + q + 1] - start[f + q] == len;
+        for (uint64_t e = 0; same && e < len; e++) same = col[start[f + q] + e] == col[start[f] + e];
+      }
+    }
+    if (same) return h;
+  }
+  return 1;
+}
+
+static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool column_runs, bool own_rows, uint64_t row_block) {
   AS_CHECK(is_supported(m, sub), "format is not supported by SHARED_MEMORY_TILE_TEMPLATE");
+  AS_CHECK(row_block >= 1 && row_block <= 4, "row blocks of 1 to 4 rows");
+  // Row blocks (row_block = b > 1, under row ownership): b consecutive rows (b divides the row's number and the
+  // row group's height) that hold the same columns are one piece of the stream -- the columns, the lane word and
+  // the x reads are those of the first row, and an element is b values, one per row.  Dense b x b blocks of a FEM
+  // matrix: 8 bytes of columns + 1 of run starts + 4 of lane word per 8 b elements.  nullptr where a block of rows
+  // does not hold the same columns in a window.
   const DenseItem &it = m.items[sub];
   const CompressedBlock &cb = *it.cb;
   const Index &bl = *cb.read_index[2];
   const uint64_t S = cb.col_slice, R = cb.row_group, B = bl.block_num, vs = (uint64_t)dtype_size(m.val_dtype);
+  if (row_block > 1 && (!own_rows || R % row_block != 0)) return nullptr;
   const std::vector<uint64_t> &row = cb.read_index[0]->index_arr.v, &col = cb.read_index[1]->index_arr.v;
   const ValVec &val = *cb.val;
   const uint64_t n = row.size(), sub_rows = it.max_row - it.min_row + 1;
@@ -302,6 +344,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   piece.reserve(n + G * kRunUnit);
   t->val_arr.reserve(n + G * kRunUnit);
   auto elem = [&](uint64_t i) { return own_rows ? (uint64_t)order[i] : i; };
+  std::vector<ValVec> other_rows(row_block - 1);  // row blocks: the values of rows 1 .. b-1 of every element
   for (uint64_t g = 0; g < G; g++) {
     group_first_run.push_back(run_slice.size());
     for (uint64_t ri = trip_first_run[g]; ri < trip_first_run[g + 1]; ri++) {
@@ -319,11 +362,13 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
         piece.push_back(cur_piece);
         t->val_arr.push_back(0.0);
       };
-      for (uint64_t i = run.begin; i < run.end; i++) {
-        const uint64_t k = elem(i), c = col[k] - col0;
-        const bool first = i == run.begin, new_row = first || row[k] != row[elem(i - 1)];
+      // one step of the loop = one element of the stream: an element of a row, or (row blocks) the elements that
+      // the rows of a block hold in one column
+      uint64_t prev_row = 0;   // first row of the piece before
+      auto take = [&](uint64_t k, uint64_t piece_row, bool first, bool new_row) {
+        const uint64_t c = col[k] - col0;
         // row ownership: a row that does not follow its predecessor directly cannot share a lane with it
-        if (own_rows && new_row && !first && row[k] != row[elem(i - 1)] + 1)
+        if (own_rows && new_row && !first && piece_row != prev_row + row_block)
           while (lcol.size() % kLaneElems) pad();
         if (column_runs) {
           if (lcol.size() % kLaneElems == 0) lane_runs = 0;
@@ -336,13 +381,48 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
           }
         }
         if (new_row) {
-          if (!own_rows) piece_target.push_back(target_of(row[k]));
+          if (!own_rows) piece_target.push_back(target_of(piece_row));
           pieces++;
-          cur_piece = own_rows ? row[k] - row0 : pieces - 1;
+          cur_piece = own_rows ? piece_row - row0 : pieces - 1;
+          prev_row = piece_row;
         }
         lcol.push_back(c);
         piece.push_back(cur_piece);
         t->val_arr.push_back(val[k]);
+      };
+      if (row_block == 1) {
+        for (uint64_t i = run.begin; i < run.end; i++) {
+          const uint64_t k = elem(i);
+          const bool first = i == run.begin;
+          take(k, row[k], first, first || row[k] != row[elem(i - 1)]);
+        }
+      } else {
+        for (uint64_t i = run.begin; i < run.end;) {
+          const uint64_t r0 = row[elem(i)];
+          if (r0 % row_block != 0 || r0 + row_block > sub_rows) return nullptr;  // the block's first row is missing here
+          uint64_t first_of[5];
+          first_of[0] = i;
+          for (uint64_t q = 0; q < row_block; q++) {
+            uint64_t j = first_of[q];
+            while (j < run.end && row[elem(j)] == r0 + q) j++;
+            first_of[q + 1] = j;
+          }
+          const uint64_t len = first_of[1] - first_of[0];
+          for (uint64_t q = 1; q < row_block; q++) {
+            if (first_of[q + 1] - first_of[q] != len) return nullptr;
+            for (uint64_t e = 0; e < len; e++)
+              if (col[elem(first_of[q] + e)] != col[elem(first_of[0] + e)]) return nullptr;
+          }
+          for (uint64_t e = 0; e < len; e++) {
+            take(elem(first_of[0] + e), r0, i == run.begin && e == 0, e == 0);
+            // the other rows' values of this element, in planes of their own until the stream is laid out
+            for (uint64_t q = 1; q < row_block; q++) {
+              other_rows[q - 1].resize(t->val_arr.size() - 1, 0.0);
+              other_rows[q - 1].push_back(val[elem(first_of[q] + e)]);
+            }
+          }
+          i = first_of[row_block];
+        }
       }
       AS_CHECK(pieces <= R && cur_piece < R, "more row pieces in a run than rows in a row group");
       while (lcol.size() % kRunUnit) {
@@ -381,7 +461,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
       for (uint64_t at = p0; at < p1; at += kLaneElems) {
         uint64_t w = piece[at];
         for (uint64_t j = 1; j < kLaneElems; j++) {
-          AS_CHECK(piece[at + j] == piece[at + j - 1] || piece[at + j] == piece[at + j - 1] + 1, "pieces must be consecutive");
+          AS_CHECK(piece[at + j] == piece[at + j - 1] || piece[at + j] == piece[at + j - 1] + row_block, "pieces must be consecutive");
           if (piece[at + j] != piece[at + j - 1]) w |= 1ull << (kNewPieceBit + j);
         }
         lane_word[at / kLaneElems] = w;
@@ -414,15 +494,23 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
   t->col_index_arr.assign(std::move(lcol), UNSIGNED_SHORT);
   // Values are read 16 bytes per lane and load; for the 64 lanes of a load to read one contiguous kilobyte,
   // the 16-byte pieces of a wavefront step are stored load by load: piece i of lane l at (i * 64 + l).
+  // Row blocks: the b rows of a lane one after the other, each in its 16-byte pieces.
   {
-    const uint64_t chunk = 16 / vs;
-    ValVec stored(padded);
+    const uint64_t chunk = 16 / vs, chunks = kLaneElems / chunk, b = row_block;
+    for (ValVec &plane : other_rows) plane.resize(padded, 0.0);
+    ValVec stored(padded * b);
     for (uint64_t u = 0; u < padded; u += kRunUnit)
       for (uint64_t lane = 0; lane < 64; lane++)
-        for (uint64_t j = 0; j < kLaneElems; j++)
-          stored[u + ((j / chunk) * 64 + lane) * chunk + j % chunk] = t->val_arr[u + lane * kLaneElems + j];
+        for (uint64_t q = 0; q < b; q++) {
+          const ValVec &plane = q == 0 ? t->val_arr : other_rows[q - 1];
+          for (uint64_t j = 0; j < kLaneElems; j++)
+            stored[u * b + ((q * chunks + j / chunk) * 64 + lane) * chunk + j % chunk] = plane[u + lane * kLaneElems + j];
+        }
     t->val_arr.swap(stored);
+    std::vector<ValVec>().swap(other_rows);
   }
+  t->scalar["row_block"] = row_block;
+  t->row_block = row_block;
 
   // the run tables are read with scalar loads, which need 32-bit entries
   auto add = [&](const char *name, std::vector<uint64_t> v, bool word) {
@@ -493,8 +581,10 @@ std::string kernel_source(const Template &t) {
   std::string s;
   s += "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(t.thread_num_in_block) + ") spmv_" + id + "(" +
        kernel_signature(t) + ")\n{\n";
+  // row blocks: a lane's loads of values cover its eight elements in each of the block's rows
+  const unsigned RB = t.scalar.count("row_block") ? (unsigned)t.sc("row_block") : 1u;
   const unsigned chunk = 16 / (unsigned)dtype_size(t.val_dtype), chunks = (unsigned)kLaneElems / chunk;
-  const std::string Cs = std::to_string(chunk), Ns = std::to_string(chunks);
+  const std::string Cs = std::to_string(chunk), Ns = std::to_string(chunks * RB);
   s += "  typedef " + vt + " val16_t __attribute__((ext_vector_type(" + Cs + ")));\n";  // 16 bytes of values
   if (t.col_runs) {
     AS_CHECK(t.arr("col_run_mask").a.dt == UNSIGNED_CHAR, "run masks must be bytes");
@@ -612,7 +702,7 @@ std::string kernel_source(const Template &t) {
     std::string c;
     c += ind + "const unsigned int unit = nz0 + k * stride, at = unit + lane * " + Ls + "u;\n";
     c += ind + "#pragma unroll\n";
-    c += ind + "for (int i = 0; i < " + Ns + "; i++) a[k][i] = as_ldnt((const val16_t *)(val_arr + unit + (i * 64u + lane) * " + Cs + "u));\n";
+    c += ind + "for (int i = 0; i < " + Ns + "; i++) a[k][i] = as_ldnt((const val16_t *)(val_arr + unit" + (RB > 1 ? " * " + std::to_string(RB) + "u" : std::string()) + " + (i * 64u + lane) * " + Cs + "u));\n";
     if (t.col_runs) {
       c += ind + "c[k] = as_ldnt((const col8_t *)(col_index_arr + (at >> 1)));\n";
       c += ind + "m[k] = as_ldnt(col_run_mask + (at >> 3));\n";
@@ -654,16 +744,42 @@ std::string kernel_source(const Template &t) {
     const std::string bit = std::to_string(1u << (kStoreBit + j)) + "u";
     // under row ownership a cell may hold the row's sum from an earlier slice: the only sum of its piece IN THIS
     // RUN is added without an atomic (nobody else touches the cell before the next barrier)
-    return "{ if (w[k] & " + bit + ") piece_sum[cell] " + std::string(t.own_rows ? "+=" : "=") + " acc; else as_lds_add(piece_sum + cell, acc); }";
+    if (RB == 1)
+      return "{ if (w[k] & " + bit + ") piece_sum[cell] " + std::string(t.own_rows ? "+=" : "=") + " acc; else as_lds_add(piece_sum + cell, acc); }";
+    // row blocks: the block's rows are neighbouring cells
+    std::string plain, atomic;
+    for (unsigned q = 0; q < RB; q++) {
+      plain += " piece_sum[cell + " + std::to_string(q) + "u] += acc" + std::to_string(q) + ";";
+      atomic += " as_lds_add(piece_sum + cell + " + std::to_string(q) + "u, acc" + std::to_string(q) + ");";
+    }
+    return "{ if (w[k] & " + bit + ") {" + plain + " } else {" + atomic + " } }";
   };
   s += "          unsigned int cell = w[k] & 0x7fffu;\n";
-  s += "          " + vt + " acc = a[k][0][0] * xv[0];\n";
-  for (unsigned j = 1; j < kLaneElems; j++) {
-    s += "          if (w[k] & " + std::to_string(1u << (kNewPieceBit + j)) + "u) { " + emit(j - 1) + " acc = 0; cell++; }\n";
-    s += "          acc += a[k][" + std::to_string(j / chunk) + "][" + std::to_string(j % chunk) + "] * xv[" + std::to_string(j) + "];\n";
+  if (RB == 1) {
+    s += "          " + vt + " acc = a[k][0][0] * xv[0];\n";
+    for (unsigned j = 1; j < kLaneElems; j++) {
+      s += "          if (w[k] & " + std::to_string(1u << (kNewPieceBit + j)) + "u) { " + emit(j - 1) + " acc = 0; cell++; }\n";
+      s += "          acc += a[k][" + std::to_string(j / chunk) + "][" + std::to_string(j % chunk) + "] * xv[" + std::to_string(j) + "];\n";
+    }
+    s += "          acc = as_wave_segmented_sum(cell, acc);\n";
+    s += "          if (as_is_segment_tail(cell)) " + emit(kLaneElems - 1) + "\n";
+  } else {
+    auto value = [&](unsigned q, unsigned j) {
+      return "a[k][" + std::to_string(q * chunks + j / chunk) + "][" + std::to_string(j % chunk) + "]";
+    };
+    for (unsigned q = 0; q < RB; q++)
+      s += "          " + vt + " acc" + std::to_string(q) + " = " + value(q, 0) + " * xv[0];\n";
+    for (unsigned j = 1; j < kLaneElems; j++) {
+      std::string zero;
+      for (unsigned q = 0; q < RB; q++) zero += " acc" + std::to_string(q) + " = 0;";
+      s += "          if (w[k] & " + std::to_string(1u << (kNewPieceBit + j)) + "u) { " + emit(j - 1) + zero + " cell += " + std::to_string(RB) + "u; }\n";
+      for (unsigned q = 0; q < RB; q++)
+        s += "          acc" + std::to_string(q) + " += " + value(q, j) + " * xv[" + std::to_string(j) + "];\n";
+    }
+    for (unsigned q = 0; q < RB; q++)
+      s += "          acc" + std::to_string(q) + " = as_wave_segmented_sum(cell, acc" + std::to_string(q) + ");\n";
+    s += "          if (as_is_segment_tail(cell)) " + emit(kLaneElems - 1) + "\n";
   }
-  s += "          acc = as_wave_segmented_sum(cell, acc);\n";
-  s += "          if (as_is_segment_tail(cell)) " + emit(kLaneElems - 1) + "\n";
   s += "        }\n      }\n    }\n  }\n}\n";
   if (t.finish_tblock_num) {
     s += "extern \"C\" __global__ void __launch_bounds__(256) spmv_" + id + "_finish(" + kernel_signature(t) + ")\n{\n";

@@ -44,7 +44,7 @@ WORKLOADS = {
     "C3": ("C3: power-law row lengths (Zipf 1.8, mean 16, max 200000), 2000000 rows, uniform columns, fp32", "power_law",
            {}, 90.0, 60.0, "sort+div64|T1@1024|T2:slice=8192,group=65536@512", 30.0),
     "C4": ("C4: FEM-like dense 3x3 blocks, 27 block columns per block row in a +-2000 band, 1000002 rows, fp64",
-           "fem_blocks", {}, 45.0, 25.0, "|T1:slice=16384,group=4096@1024,runs,own", 35.0),
+           "fem_blocks", {}, 45.0, 25.0, "|T1:slice=16384,group=4092@1024,runs,own,blk3", 35.0),
     "C5": ("C5: 8000000 rows of 1-3 elements + 800 rows of 50000-1000000 elements, uniform columns, fp64",
            "extreme_irregular", {"target_nnz": 60_000_000}, 150.0, 75.0,
            "sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256", 45.0),
@@ -130,14 +130,18 @@ def build_pinned(m, pin):
         skel, _, kw = spec.partition(":")
         kw = {k: int(x) for k, x in (p.split("=") for p in filter(None, kw.split(",")))}
         words = [x for x in launch.split(",") if x]
-        chosen.append((SK.apply_skeleton(m, s, skel, **kw)[0], [int(x) for x in words if x.isdigit()], "runs" in words, "own" in words))
+        blocks = [int(x[3:]) for x in words if x.startswith("blk")]
+        chosen.append((SK.apply_skeleton(m, s, skel, **kw)[0], [int(x) for x in words if x.isdigit()], "runs" in words, "own" in words,
+                       blocks[0] if blocks else 0))
     b = A.Builder(m)
-    for s, (tp, launch, runs, own) in enumerate(chosen):
+    for s, (tp, launch, runs, own, blocks) in enumerate(chosen):
         b.set_template(s, tp)
         if runs and not b.set_column_runs(s):
             raise SystemExit("bench.py: the column-run form does not apply to strip %d" % s)
         if own and not b.set_row_ownership(s):
             raise SystemExit("bench.py: row ownership does not apply to strip %d" % s)
+        if blocks and not b.set_row_blocks(s, blocks):
+            raise SystemExit("bench.py: the rows of strip %d do not come in blocks of %d" % (s, blocks))
         if launch:
             b.set_launch(s, thread_num_in_block=launch[0], vec_width=launch[1] if len(launch) > 1 else 0)
     b.set_serial_launch(serial)
@@ -247,6 +251,7 @@ def measure(key, steps, warmup, tune_seconds, pin, cpu_seconds, copy_calibration
                    "template": templates, "launch": launches,
                    "columns": [column_form(s) for s in range(int(res.n_sub))],
                    "rows_owned": ["run_row_group" in b.describe(s)["arrays"] for s in range(int(res.n_sub))],
+                   "row_block": [int(b.describe(s).get("row_block", 1)) for s in range(int(res.n_sub))],
                    "clears_y": b.clears_y(), "graph_hash": graph_hash},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
@@ -282,7 +287,7 @@ def per_matrix_entry(key, full):
     e = {"workload": key, "gflops": full["value"], "ms_per_step": full["ms_per_step"], "steps": full["steps"],
          "dtype": full["dtype"], "rows": full["config"]["rows"], "nnz": full["config"]["nnz"],
          "graph": {k: full["config"][k] for k in ("dense_strategy", "sub_matrices", "template", "launch", "columns",
-                                                   "rows_owned", "clears_y", "graph_hash", "pinned")},
+                                                   "rows_owned", "row_block", "clears_y", "graph_hash", "pinned")},
          "roofline": {k: full["roofline"][k] for k in ("frac", "achieved", "kernel", "kernel_us", "algorithmic_bytes",
                                                        "csr_floor_bytes", "csr_floor_frac", "traffic", "traffic_profile")},
          "whole_spmv": full["whole_spmv"], "kernels": full["kernels"], "tuning": full["tuning"], "check": full["check"]}

@@ -245,6 +245,14 @@ int as_builder_set_column_runs(as_builder *b, int64_t sub);
  * move more than a quarter of the element stream, or row groups too few or too uneven to fill the device),
  * -1 error. */
 int as_builder_set_row_ownership(as_builder *b, int64_t sub);
+/* No counterpart in the reference.  Tile template under row ownership only: where the rows of the sub-matrix come
+ * in blocks of `rows_per_block` (2, 3 or 4) consecutive rows that hold the same columns (the dense blocks of a FEM
+ * matrix), the template is built again with a block of rows as one piece of the stream: the columns, the lane
+ * word and the reads of x are those of the block's first row, an element is one value per row.  The row group's
+ * height must be a multiple of the block.  1 = done (upload again; launch setting, column-run form and row
+ * ownership are kept), 0 = nothing changed (another template or form, rows that do not come in such blocks),
+ * -1 error. */
+int as_builder_set_row_blocks(as_builder *b, int64_t sub, int rows_per_block);
 int as_builder_get_launch(as_builder *b, int64_t sub, long out[4]);
 /* arrays of a template by upstream field name (what store_template_data writes to data_source/<id>/<name>).
  * "col_index_arr" and every metadata array here, "val_arr" through as_template_get_f64.

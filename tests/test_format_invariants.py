@@ -184,6 +184,8 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
     arr = {k: np.asarray(a[0]).astype(np.int64) for k, a in t["arrays"].items()}
     val = np.asarray(t["val_arr"][0] if isinstance(t["val_arr"], tuple) else t["val_arr"], np.float64)
     own_rows = "run_row_group" in arr   # row ownership: cells are rows of the run's row group, kept across its runs
+    rb = int(t["scalars"].get("row_block", 1))   # row blocks: an element is one value for each of rb neighbouring rows
+    assert rb == 1 or own_rows
     gfr, nzb, word, yrow, lcol = (arr["group_first_run"], arr["run_nz_begin"], arr["lane_word"],
                                   arr["y_row_index"], arr["col_index_arr"])
     # the first column of the stretch of x a run reads: a slice of the format's grid, or (row ownership) a window
@@ -216,15 +218,20 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
             decoded[:, j] = np.where(opens == 1, np.where(run < 4, starts[lanes, np.minimum(run, 3)], 0), decoded[:, j - 1] + 1)
         lcol = decoded.reshape(-1)
     assert gfr[0] == 0 and gfr[-1] == len(rs) and (np.diff(gfr) > 0).all() and (np.diff(nzb) > 0).all()
-    assert nzb[-1] * 512 == len(lcol) == len(val) == 8 * len(word) and (lcol < slice_width).all()
+    assert nzb[-1] * 512 * rb == len(lcol) * rb == len(val) == 8 * len(word) * rb and (lcol < slice_width).all()
     if not own_rows:
         assert rpb[0] == 0 and rpb[-1] == len(target) and (np.diff(rpb) > 0).all() and (np.diff(rpb) <= group).all()
     through_scratch = t["scalars"]["is_atom_add"] == 0 and not own_rows
     group_cells = {}
     # values are stored 16 bytes per lane and load: piece i of lane l of a wavefront step at (i * 64 + l)
+    # (row blocks: the rb rows of a lane one after the other, each in its 16-byte pieces: val[q] = the values of row q)
     j, lane = np.meshgrid(np.arange(8), np.arange(64))
-    where = ((j // chunk) * 64 + lane) * chunk + j % chunk       # [lane, j] -> place inside the step
-    val = val.reshape(-1, 512)[:, where.reshape(-1)].reshape(-1)
+    steps = val.reshape(-1, 512 * rb)
+    val_rows = []
+    for q in range(rb):
+        where = ((q * (8 // chunk) + j // chunk) * 64 + lane) * chunk + j % chunk    # [lane, j] -> place inside the step
+        val_rows.append(steps[:, where.reshape(-1)].reshape(-1))
+    val = val_rows[0]
     y = np.zeros(int(yrow.max()) + 1)
     flagged = plain = 0
     for run in range(len(rs)):
@@ -235,45 +242,45 @@ def _emulate_tile_template(t, slice_width, group, sub_rows, x, chunk=4):
             cells = np.zeros(rpb[run + 1] - rpb[run])
         touched = np.zeros(len(cells), np.int64)
         assert (rs[run] + lcol[k0:k1] < len(x)).all()            # padding included: the kernel reads x there
-        prod = val[k0:k1] * x[rs[run] + lcol[k0:k1]]
+        prods = [vq[k0:k1] * x[rs[run] + lcol[k0:k1]] for vq in val_rows]
         for u in range(0, k1 - k0, 512):                         # one wavefront step
             w = word[(k0 + u) // 8:(k0 + u) // 8 + 64]
             first = w & 0x7fff
             new_piece = (w[:, None] >> (14 + np.arange(1, 8))[None, :]) & 1
             store = (w[:, None] >> (22 + np.arange(8))[None, :]) & 1
-            final = first + new_piece.sum(1)
+            final = first + rb * new_piece.sum(1)
             step = first[1:] - final[:-1]
             if own_rows:
-                assert (step >= 0).all()                         # a lane may skip rows that have no element in the slice
+                assert (step >= 0).all() and (first % rb == 0).all()   # a lane may skip rows that have no element in the slice
             else:
                 assert ((step == 0) | (step == 1)).all()          # the next lane goes on with the piece or starts the next one
-            carry = 0.0                                          # the segmented sum over the lanes' last pieces
+            carry = np.zeros(rb)                                 # the segmented sum over the lanes' last pieces
             for lane in range(64):
-                cell, acc = first[lane], 0.0
+                cell, acc = first[lane], np.zeros(rb)
 
                 def emit(j):
                     nonlocal flagged, plain
-                    assert cell < len(cells)
+                    assert cell + rb <= len(cells)
                     if store[lane, j]:
                         assert touched[cell] == 0                # the only sum of this piece (in this run)
-                        cells[cell] = cells[cell] + acc if own_rows else acc
+                        cells[cell:cell + rb] = cells[cell:cell + rb] + acc if own_rows else acc
                         touched[cell] = -1
                         flagged += 1
                     else:
                         assert touched[cell] >= 0
-                        cells[cell] += acc
+                        cells[cell:cell + rb] += acc
                         touched[cell] += 1
                         plain += 1
                 for j in range(8):
                     if j and new_piece[lane, j - 1]:
                         emit(j - 1)
-                        cell, acc = cell + 1, 0.0
-                    acc += prod[u + lane * 8 + j]
+                        cell, acc = cell + rb, np.zeros(rb)
+                    acc = acc + np.array([p[u + lane * 8 + j] for p in prods])
                 if lane and final[lane - 1] == final[lane]:
-                    acc += carry
+                    acc = acc + carry
                 if lane == 63 or final[lane + 1] != final[lane]:
                     emit(7)
-                    carry = 0.0
+                    carry = np.zeros(rb)
                 else:
                     carry = acc
         if own_rows:
@@ -411,6 +418,63 @@ def test_tile_template_under_row_ownership(vdt, chunk, sort, runs):
     b = A.Builder(m)
     b.set_template(0, SK.apply_skeleton(m, 0, "S1", m=64)[0])
     assert not b.set_row_ownership(0)
+
+
+@pytest.mark.parametrize("vdt,chunk", [(K.FLOAT, 4), (K.DOUBLE, 2)], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("runs", [False, True], ids=["plain", "runs"])
+def test_tile_template_with_row_blocks(vdt, chunk, runs):
+    """set_row_blocks on a matrix of dense 3 x 3 blocks under row ownership: the three rows of a block row hold the
+    same columns and become one piece of the stream -- one set of columns and lane words, three values per element,
+    a third of the stream's elements -- and walking the arrays the way the kernel does gives the same y.  Turned
+    down where the row group's height is not a multiple of three, without row ownership, for blocks of another
+    height, and where a row of a block differs from the others."""
+    from alphasparse_amd import skeletons as SK
+    rows, cols, r, c, v, x = S.fem_blocks(1000, 27, 60, seed=5)
+    vv = np.float32(v).astype(np.float64) if vdt == K.FLOAT else v.astype(np.float64)
+    yref = np.zeros(rows)
+    np.add.at(yref, np.asarray(r, np.int64), vv * x[np.asarray(c, np.int64)])
+
+    def build(matrix_rows=(rows, r, c, v), group=96):
+        n, rr, cc, vals = matrix_rows
+        m = A.Matrix.from_coo(n, cols, rr, cc, vals.astype(np.float64), vdt, wave=64)
+        m.execute_strategy(K.COMPRESS_NONE)
+        tp = SK.apply_skeleton(m, 0, "T1", slice=500, group=group, b=1000)[0]
+        b = A.Builder(m)
+        b.set_template(0, tp, compress=False)
+        b.set_launch(0, thread_num_in_block=256)
+        return b
+    b = build()
+    assert not b.set_row_blocks(0, 3)                                    # not before row ownership
+    if runs:
+        assert b.set_column_runs(0)
+    assert b.set_row_ownership(0)
+    before = b.template_dump(0)
+    assert not b.set_row_blocks(0, 2) and not b.set_row_blocks(0, 4)     # 96 = 4 x 24, but the blocks are 3 rows high
+    assert b.set_row_blocks(0, 3) and not b.set_row_blocks(0, 3)         # the second call finds the form in place
+    t = b.template_dump(0)
+    assert t["scalars"]["row_block"] == 3 and "run_row_group" in t["arrays"] and ("col_run_mask" in t["arrays"]) == runs
+    assert len(t["val_arr"]) <= 1.25 * len(before["val_arr"])            # the same values; a run is padded to 512 elements of 3 values
+    assert len(t["arrays"]["lane_word"][0]) * 2.5 <= len(before["arrays"]["lane_word"][0])   # a third of the lanes
+    assert not b.clears_y() and b.get_launch(0)["thread_num_in_block"] == 256
+    y, flagged, plain = _emulate_tile_template(t, 500, 96, rows, x.astype(np.float64), chunk=chunk)
+    assert np.allclose(y, yref, rtol=1e-12, atol=1e-12) and flagged > 0
+    src = b.kernel_source()
+    assert "acc2" in src and "cell += 3u" in src and ("col_run_mask" in src) == runs
+    if not runs:                                                         # the column-run form on top keeps the blocks
+        assert b.set_column_runs(0)
+        t2 = b.template_dump(0)
+        assert t2["scalars"]["row_block"] == 3 and "col_run_mask" in t2["arrays"]
+        y2 = _emulate_tile_template(t2, 500, 96, rows, x.astype(np.float64), chunk=chunk)[0]
+        assert np.allclose(y2, yref, rtol=1e-12, atol=1e-12)
+    # a row group height that the block does not divide
+    b = build(group=100)
+    assert b.set_row_ownership(0) and not b.set_row_blocks(0, 3)
+    # one element taken out of one row: its block no longer holds the same columns in its three rows
+    keep = np.ones(len(r), bool)
+    keep[np.flatnonzero(np.asarray(r) == 301)[5]] = False
+    b = build((rows, np.asarray(r)[keep], np.asarray(c)[keep], np.asarray(v)[keep]))
+    assert b.set_row_ownership(0) and not b.set_row_blocks(0, 3)
+    assert b.template_dump(0)["scalars"].get("row_block", 1) == 1        # nothing changed
 
 
 def test_tile_template_stores_fp64_values_two_per_lane_and_load():

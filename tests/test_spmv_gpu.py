@@ -344,6 +344,60 @@ def test_tile_template_under_row_ownership(gpu, vdt, sort, runs, threads):
         b.close()
 
 
+@pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("runs", [False, True], ids=["columns", "runs"])
+@pytest.mark.parametrize("threads", [1024, 256])
+def test_tile_template_with_row_blocks(gpu, vdt, runs, threads):
+    """The tile kernel under row ownership with blocks of rows as pieces (the rows of a block hold the same columns;
+    one set of columns and lane words, one value per row and element): same y as the CPU CSR oracle on matrices of
+    dense 3 x 3, 2 x 2 and 4 x 4 blocks, with row groups that meet one, two or three windows of x, a last row group
+    shorter than the others, block rows at the ragged edge of the band; y holds NaN before the call."""
+    def blocks_of(height, block_rows, per_row, band, seed):
+        # dense height x height blocks from the 3 x 3 generator's block pattern
+        rows3, cols3, r3, c3, v3, _ = S.fem_blocks(block_rows, per_row, band, seed=seed)
+        br, bc = np.asarray(r3[::9]) // 3, np.asarray(c3[::9]) // 3              # one entry per block, row-major
+        blocks = np.unique(br.astype(np.int64) * block_rows + bc)
+        br, bc = blocks // block_rows, blocks % block_rows
+        i, j = np.meshgrid(np.arange(height), np.arange(height), indexing="ij")
+        order = np.lexsort((bc, br))
+        br, bc = br[order], bc[order]
+        # row-major over the whole matrix: block row, row inside the block, block column, column inside the block
+        rr, cc = [], []
+        for q in range(height):
+            rr.append(np.repeat(br * height + q, height))
+            cc.append((bc[:, None] * height + np.arange(height)[None, :]).ravel())
+        rr, cc = np.concatenate(rr), np.concatenate(cc)
+        order = np.lexsort((cc, rr))
+        rr, cc = rr[order], cc[order]
+        rng = np.random.default_rng(seed)
+        n = block_rows * height
+        return n, n, rr.astype(np.uint64), cc.astype(np.uint64), rng.uniform(-1, 1, len(rr)), rng.uniform(-1, 1, n)
+    for height, gen, slice_width, group in ((3, lambda: S.fem_blocks(3000, 27, 400), 4000, 252),
+                                            (3, lambda: S.fem_blocks(1000, 9, 60, seed=3), 500, 96),
+                                            (2, lambda: blocks_of(2, 3000, 27, 200, 7), 1000, 256),
+                                            (4, lambda: blocks_of(4, 900, 9, 50, 8), 700, 128)):
+        rows, cols, r, c, v, x = gen()
+        npd = NP[vdt]
+        v, x = v.astype(npd), x.astype(npd)
+        y_ref, mag = oracle_y(rows, r, c, v, x)
+        m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+        m.execute_strategy(K.COMPRESS_NONE)
+        tp = SK.apply_skeleton(m, 0, "T1", slice=slice_width, group=group, b=4096)[0]
+        b = A.Builder(m)
+        b.set_template(0, tp)
+        if runs:
+            assert b.set_column_runs(0)
+        assert b.set_row_ownership(0), (rows, slice_width, group)
+        assert b.set_row_blocks(0, height), (rows, slice_width, group, height)
+        b.set_launch(0, thread_num_in_block=threads)
+        b.compile().upload(gpu)
+        print("case: row blocks", height, rows, cols, len(r), slice_width, group, threads, runs, flush=True)
+        assert not b.clears_y() and "cell += %du" % height in b.kernel_source()
+        assert_y(b.spmv(x), y_ref, mag, npd, "tile template, row blocks")
+        assert_y(b.spmv_device(x), y_ref, mag, npd, "tile template, row blocks, y = NaN before the call")
+        b.close()
+
+
 @pytest.mark.parametrize("position", [K.END_PADDING, K.TOP_PADDING], ids=["end", "top"])
 @pytest.mark.parametrize("skel,kw", [("S5", {}), ("S1", {"m": 64}), ("T1", {"slice": 1024, "group": 512, "b": 2048})],
                          ids=["S5", "S1", "T1"])
