@@ -59,7 +59,8 @@ PROFILE_OF = {"C2": "profiles/spmv_ell_c2_laplacian_hbm_traffic.txt", "C3": "pro
 MEASURED_TRAFFIC = {
     "ff84531ca565a608": 117580800,    # C2, ELL kernel in diagonal form (pin S5,256,1,dia)
     "e9afcd580f447551": 197734396,    # C3, tile kernel of the long strip + its finish (pin sort+div64|T1@1024|T2:slice=8192,group=65536@512)
-    "3b570d6d4c746c50": 803162829,    # C4, tile kernel, column runs under row ownership (pin |T1:slice=16384,group=4096@1024,runs,own)
+    "dad308d7a3b7a127": 711696691,    # C4, tile kernel, column runs, row ownership, blocks of 3 rows (pin |T1:slice=16384,group=4092@1024,runs,own,blk3)
+    "3b570d6d4c746c50": 803162829,    # C4, the same without row blocks (pin |T1:slice=16384,group=4096@1024,runs,own)
     "b9791554820cbb6f": 688027956,    # C5, product-bin kernel, both passes (pin sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256)
 }
 
