@@ -65,6 +65,29 @@ def test_search_result_is_correct_and_reported(gpu, name):
     b.close()
 
 
+def test_search_stores_a_block_matrix_by_blocks_of_rows(gpu):
+    """A banded matrix of dense 3 x 3 blocks whose x does not fit the L2 cache of an XCD (540,000 columns, fp64): the
+    search offers the tile skeleton with row groups of whole blocks, and the tile template wins in its column-run
+    form under row ownership with blocks of three rows as pieces.  The report says so, and the graph rebuilt from the
+    report's nodes gives A x."""
+    rows, cols, r, c, v, x = S.fem_blocks(180000, 9, 2000, seed=12)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.DOUBLE, wave=64)
+    res = A.find_best_graph(m, total_time_s=30.0, device=gpu, timed_region_ms=5.0, only_dense_strategy=1)
+    print("block matrix: best %.1f GFLOP/s, %d candidates, %.1f s" % (res.gflops, res.candidates, res.seconds), flush=True)
+    assert res.failed_candidates == 0
+    rep = res.report
+    assert "kernel_node_type:SHARED_MEM_X_SLICE" in rep, rep
+    assert "col_index_runs:1\n" in rep and "y_rows_owned:1\n" in rep and "row_block:3\n" in rep, rep
+    assert re.search(r"row_group_size:(\d+)", rep) and int(re.search(r"row_group_size:(\d+)", rep).group(1)) % 3 == 0
+    b = _check_best(res, rows, r, c, v, x, gpu, np.float64)
+    d = b.describe(0)
+    assert d["row_block"] == 3 and "run_row_group" in d["arrays"] and not b.clears_y()
+    y_ref, mag = _oracle(rows, r, c, v, x)
+    rel, ratio, tol = O.check_y(b.spmv_device(x), y_ref, mag, np.float64)
+    assert rel <= tol and ratio <= 1.0, (rel, ratio)
+    b.close()
+
+
 def test_configuration_1_at_its_stated_shape(gpu):
     """Benchmark configuration 1 exactly as stated: 4096 x 4096, 8 elements in every row at seeded uniform columns
     (32,768 elements), values and x in [-1, 1], fp32.  A short search, then the rebuilt best graph against the CPU

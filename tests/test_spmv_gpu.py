@@ -545,7 +545,7 @@ def _full_c3():
 
 
 def _full_c4():
-    return S.fem_blocks(), K.DOUBLE, None, ("T1", {"slice": 16384, "group": 4096}, 1024)
+    return S.fem_blocks(), K.DOUBLE, None, ("T1", {"slice": 16384, "group": 4092}, 1024)
 
 
 def _full_c5():
@@ -557,8 +557,8 @@ def _full_c5():
 def test_full_size_tile_and_product_bin_graphs(gpu, make, capsys):
     """The benchmark matrices at their real size through the graphs the search returns for them -- C3 (2 M rows,
     32 M elements, fp32) and C5 (8 M rows, 60 M elements, fp64): coarse sort, two row strips, the tile kernel on the
-    long rows and the product-bin kernel on the others; C4 (1 M rows, 81 M elements, fp64): the tile kernel in its
-    column-run form on the whole matrix.  y against the CPU CSR oracle, and two properties that do not depend on the
+    long rows and the product-bin kernel on the others; C4 (1 M rows, 81 M elements, fp64): the tile kernel on the
+    whole matrix, column-run form under row ownership with blocks of three rows as pieces.  y against the CPU CSR oracle, and two properties that do not depend on the
     size: x = 1 gives the row sums of the values, and A (2 x - 3 z) = 2 A x - 3 A z within the rounding of the row.
     Most of a case's time is the generation of the matrix: the phases are announced past the capture."""
     def say(what):
@@ -583,15 +583,16 @@ def test_full_size_tile_and_product_bin_graphs(gpu, make, capsys):
         b.set_template(s, tp)
         b.set_launch(s, thread_num_in_block=strips[s][2])
     if not long_strip:
-        assert b.set_column_runs(0)                              # C4: dense 3 x 3 blocks
+        # C4, dense 3 x 3 blocks: column runs, whole row groups per workgroup, blocks of three rows as pieces
+        assert b.set_column_runs(0) and b.set_row_ownership(0) and b.set_row_blocks(0, 3)
     b.set_serial_launch(True)
     b.compile().upload(gpu)
     say("on the device: y against the oracle, row sums, linearity")
     y_ref, mag = oracle_y(rows, r, c, v, x)
     y1 = b.spmv(x)
     assert_y(y1, y_ref, mag, npd, make.__name__)
-    # C3 and C5 (a sorted tile strip + a product-bin strip) store every row once: no clear; C4 adds into y
-    assert b.clears_y() == (not long_strip)
+    # every row is stored once in all three graphs (finish kernels, or the row groups' owners): no clear of y
+    assert not b.clears_y()
     assert_y(b.spmv_device(x), y_ref, mag, npd, make.__name__ + " (y = NaN before the call)")
     eps = np.finfo(npd).eps
     off = np.concatenate([[0], np.cumsum(np.bincount(np.asarray(r, np.int64), minlength=rows))])
