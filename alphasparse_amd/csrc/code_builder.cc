@@ -517,11 +517,13 @@ void time_spmv(Builder &b, uint64_t reps, bool sync_each, float &time_ms, float 
   // The timed step is the product call: what launch_spmv issues, the clear of y included where the graph needs
   // it.  Measurements of one sub-matrix's kernels alone (only_sub) are kernel times: y is cleared once, before.
   const bool clear_each = b.only_sub < 0 && y_needs_clear(b);
-  zero_y(b, b.y.ptr);
-  HIPL(as_hip_stream_sync(b.main_stream));
+  if (b.only_sub >= 0) {
+    zero_y(b, b.y.ptr);
+    HIPL(as_hip_stream_sync(b.main_stream));
+  }
   HIPL(as_hip_event_record(b.t0, b.main_stream));
   for (uint64_t r = 0; r < reps; r++) {
-    if (clear_each && r > 0) zero_y(b, b.y.ptr);
+    if (clear_each) zero_y(b, b.y.ptr);
     launch_kernels(b, b.x.ptr, b.y.ptr);
     if (sync_each) HIPL(as_hip_stream_sync(b.main_stream));
   }
