@@ -658,6 +658,30 @@ def test_finish_of_a_tile_strip_carried_by_the_next_strips_kernel(gpu, vdt):
     assert "carried_sum" not in b.kernel_source()
     assert_y(b.spmv_device(x), y_ref, mag, npd, "concurrent streams")
     b.close()
+    # rows that already come longest first: the sort leaves them where they are, the tile strip's places in y are
+    # a closed form (no array is passed) and the carrying kernel computes them
+    order = np.argsort(-np.bincount(np.asarray(r, np.int64), minlength=rows), kind="stable")
+    new_row = np.empty(rows, np.int64)
+    new_row[order] = np.arange(rows)
+    r2 = new_row[np.asarray(r, np.int64)]
+    keep = np.lexsort((np.asarray(c, np.int64), r2))
+    r2, c2, v2 = r2[keep].astype(np.uint64), np.asarray(c)[keep], v[keep]
+    y_ref, mag = oracle_y(rows, r2, c2, v2, x)
+    m = A.Matrix.from_coo(rows, cols, r2, c2, v2.astype(np.float64), vdt, wave=64)
+    m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+    m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (16, 16, 2, 0))
+    m.execute_strategy(K.COMPRESS_NONE)
+    b = A.Builder(m)
+    b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=1024, group=512, b=2048)[0])
+    b.set_template(1, SK.apply_skeleton(m, 1, "T2", slice=1024, group=4096, b=2048)[0])
+    b.set_serial_launch(True)
+    b.compile().upload(gpu)
+    src = b.kernel_source()
+    print("case: carried finish, rows already sorted; places passed as an array:", "carried_place" in src, flush=True)
+    assert b.finish_carrier(0) == 1 and "carried_sum" in src
+    assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, rows already in sorted order")
+    assert_y(b.spmv_device(z), *oracle_y(rows, r2, c2, v2, z), npd, "carried finish, rows already in sorted order, second call")
+    b.close()
 
 
 def test_missing_library_is_an_error_not_a_fallback():
