@@ -28,6 +28,17 @@
 // columns are the previous one plus 1.  That is 9 bytes of columns per lane instead of 16 (fp64 element: 9.625
 // bytes instead of 10.5).  A lane that would need a fifth run is closed with zero-valued elements and the run
 // opens the next lane; a run start beyond the fourth decodes as column 0, which is where padding points.
+//
+// Row ownership (init_variant(..., own_rows = true)): where the matrix has many row groups that each meet few
+// columns (banded matrices), a trip is a whole number of row groups and the elements are taken row group by row
+// group, inside a group window by window of x (a window starts at the group's first column not yet covered and is
+// col_slice columns wide), inside a window row by row.  The LDS cell of a row is its place in the group and lives
+// across the group's runs; at the end of a group the workgroup stores the group's rows to y: no atomics into y,
+// no table of places, no scratch vector, no finish kernel, no clear of y.
+//
+// Row blocks (init_variant(..., row_block = b), under row ownership): where b consecutive rows hold the same
+// columns (the dense b x b blocks of a FEM matrix), a block of rows is one piece: columns, lane word and reads of
+// x are those of its first row, an element is b values, and a lane adds into b sums.
 #include "templates.hpp"
 
 namespace asx {

@@ -237,9 +237,9 @@ int as_builder_set_diagonal_columns(as_builder *b, int64_t sub);
  * by 2 %), -1 error. */
 int as_builder_set_column_runs(as_builder *b, int64_t sub);
 /* No counterpart in the reference.  Tile template (AS_SHARED_MEMORY_TILE_TEMPLATE) only: the template is built
- * again under row ownership -- the tiles are taken row group by row group, every row group belongs to one
- * workgroup, which keeps the group's row sums in LDS across the column slices and stores the rows to y at the end:
- * no atomics, no table of places, no clear of y.  For matrices of many row groups that meet few column slices
+ * again under row ownership -- the elements are taken row group by row group (inside a group window by window of
+ * x, from the group's own first column), every row group belongs to one workgroup, which keeps the group's row
+ * sums in LDS across its windows and stores the rows to y at the end: no atomics, no table of places, no clear of y.  For matrices of many row groups that meet few column slices
  * each (banded matrices).  1 = done (upload again; the launch setting and the column-run form are kept), 0 =
  * nothing changed (another template, the form is in place, a column band of the matrix, slice copies that would
  * move more than a quarter of the element stream, or row groups too few or too uneven to fill the device),
