@@ -1001,59 +1001,83 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
     for (uint64_t rate : {4, 8, 16})
       if (row_div_position_acc_to_exponential_increase_row_nnz_range({shortest_row, longest_row}, low, 2048, rate).size() > 2)
         one_strip_only = false;
+  // Upstream's order is 1, 2, 3.  Where the vector is larger than an XCD's L2 cache and the longest row is far above
+  // the average -- the matrices whose best graph is a coarse sort and two row strips -- strategy 3 goes first: its
+  // winner is then known early (it is what a caller waits for), and it bounds what strategies 1 and 2 still sweep.
+  // It leaves them a fifth of the budget.
+  const bool sort_first = opt.only_dense_strategy == 0 && !one_strip_only &&
+                          in.col_index_max + 1 > (4ull << 20) / (in.val_dtype == DOUBLE ? 8 : 4) &&
+                          longest_row >= 64 * std::max<uint64_t>(1, in.row.size() / row_len.size());
   // strategy 1: INPUT -> COMPRESS (a tenth of the budget, :5092)
-  if (opt.only_dense_strategy == 0 || opt.only_dense_strategy == 1) {
-    c.log("== dense strategy 1: INPUT -> COMPRESS" + c.stamp());
-    BestGraph g;
-    if (search_dense_strategy(c, in, {input, compress}, opt.only_dense_strategy == 1 || one_strip_only ? T : T / 10, g)) consider(g, "strategy1");
-  }
-  // strategy 2: INPUT -> ROW_DIV by exponential row-length bands -> COMPRESS (a quarter of what is left, :5156)
-  if ((opt.only_dense_strategy == 0 || opt.only_dense_strategy == 2) && now_s() < T && !one_strip_only) {
-    c.log("== dense strategy 2: INPUT -> DENSE_ROW_DIV -> COMPRESS" + c.stamp());
-    c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
-    StrategyNode div = make_strategy(DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY, 32, 2048, 4, 0);
-    const size_t strips = strips_of(row_len, 32, 2048, 4).size();
-    const bool usable = strips >= 2 && strips <= 4;
-    BestGraph g;
-    if (usable && search_dense_strategy(c, in, {input, div, compress}, opt.only_dense_strategy == 2 ? T : (T - now_s()) / 4, g))
-      consider(g, "strategy2");
-    else if (!usable) c.log("strategy 2 skipped: row division yields 1 or more than 4 strips");
-  }
-  // strategy 3: INPUT -> COARSE_SORT -> ROW_DIV(low x rate) -> COMPRESS (the rest, :4579-5039)
-  if ((opt.only_dense_strategy == 0 || opt.only_dense_strategy == 3) && now_s() < T && !one_strip_only) {
-    c.log("== dense strategy 3: INPUT -> DENSE_ROW_COARSE_SORT -> DENSE_ROW_DIV -> COMPRESS" + c.stamp());
-    StrategyNode sort = make_strategy(DENSE_ROW_COARSE_SORT_FIXED_PARAM_STRATEGY, 1);
-    BestGraph best3;
-    // (lowest, highest, rate) of the row-length bands.  First two strips only -- rows of at least
-    // `lowest` elements and the rest -- which is what the LDS-tile kernel wants when x is larger
-    // than an XCD's L2 cache; then the upstream grid 512/128/32 x 4/8/16 with bands up to 2048.
-    std::vector<std::array<long, 3>> bands;
-    if (in.col_index_max + 1 > (4ull << 20) / (in.val_dtype == DOUBLE ? 8 : 4))
-      for (long low : {16, 64, 256}) bands.push_back({low, low, 2});
-    for (long low : {512, 128, 32})
-      for (long rate : {4, 8, 16}) bands.push_back({low, 2048, rate});
-    std::vector<std::vector<uint64_t>> seen;
-    // A row division is a step of this level's search, and like the levels below it ends after steps in a row
-    // that bring nothing (three here: a step costs seconds on a large matrix, not milliseconds).
-    int struggle = 0;
-    for (size_t bi = 0; bi < bands.size() && now_s() < T; bi++) {
-      StrategyNode div = make_strategy(DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY, bands[bi][0], bands[bi][1], bands[bi][2], 0);
-      std::vector<uint64_t> cut = strips_of(sorted_len, bands[bi][0], bands[bi][1], bands[bi][2]);
-      if (cut.size() > 4 || cut.size() < 2) continue;
-      if (std::find(seen.begin(), seen.end(), cut) != seen.end()) continue;  // same strips as an earlier combination
-      seen.push_back(cut);
-      c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
+  auto strategy1 = [&]() {
+    if ((opt.only_dense_strategy == 0 || opt.only_dense_strategy == 1) && now_s() < T) {
+      c.log("== dense strategy 1: INPUT -> COMPRESS" + c.stamp());
+      if (sort_first) c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
       BestGraph g;
-      double budget = (T - now_s()) / 2;
-      if (search_dense_strategy(c, in, {input, sort, div, compress}, budget, g) && g.gflops > best3.gflops) {
-        best3 = g;
-        struggle = 0;
-      } else if (best3.gflops > 0 && ++struggle >= 3) {
-        c.log("three row divisions in a row without an improvement: strategy 3 ends" + c.stamp());
-        break;
-      }
+      if (search_dense_strategy(c, in, {input, compress}, opt.only_dense_strategy == 1 || one_strip_only ? T : T / 10, g)) consider(g, "strategy1");
     }
-    if (best3.gflops > 0) consider(best3, "strategy3");
+  };
+  // strategy 2: INPUT -> ROW_DIV by exponential row-length bands -> COMPRESS (a quarter of what is left, :5156)
+  auto strategy2 = [&]() {
+    if ((opt.only_dense_strategy == 0 || opt.only_dense_strategy == 2) && now_s() < T && !one_strip_only) {
+      c.log("== dense strategy 2: INPUT -> DENSE_ROW_DIV -> COMPRESS" + c.stamp());
+      c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
+      StrategyNode div = make_strategy(DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY, 32, 2048, 4, 0);
+      const size_t strips = strips_of(row_len, 32, 2048, 4).size();
+      const bool usable = strips >= 2 && strips <= 4;
+      BestGraph g;
+      if (usable && search_dense_strategy(c, in, {input, div, compress}, opt.only_dense_strategy == 2 ? T : (T - now_s()) / 4, g))
+        consider(g, "strategy2");
+      else if (!usable) c.log("strategy 2 skipped: row division yields 1 or more than 4 strips");
+    }
+  };
+  // strategy 3: INPUT -> COARSE_SORT -> ROW_DIV(low x rate) -> COMPRESS (the rest, :4579-5039)
+  auto strategy3 = [&]() {
+    if ((opt.only_dense_strategy == 0 || opt.only_dense_strategy == 3) && now_s() < T && !one_strip_only) {
+      c.log("== dense strategy 3: INPUT -> DENSE_ROW_COARSE_SORT -> DENSE_ROW_DIV -> COMPRESS" + c.stamp());
+      StrategyNode sort = make_strategy(DENSE_ROW_COARSE_SORT_FIXED_PARAM_STRATEGY, 1);
+      BestGraph best3;
+      // (lowest, highest, rate) of the row-length bands.  First two strips only -- rows of at least
+      // `lowest` elements and the rest -- which is what the LDS-tile kernel wants when x is larger
+      // than an XCD's L2 cache; then the upstream grid 512/128/32 x 4/8/16 with bands up to 2048.
+      std::vector<std::array<long, 3>> bands;
+      if (in.col_index_max + 1 > (4ull << 20) / (in.val_dtype == DOUBLE ? 8 : 4))
+        for (long low : {16, 64, 256}) bands.push_back({low, low, 2});
+      for (long low : {512, 128, 32})
+        for (long rate : {4, 8, 16}) bands.push_back({low, 2048, rate});
+      std::vector<std::vector<uint64_t>> seen;
+      // A row division is a step of this level's search, and like the levels below it ends after steps in a row
+      // that bring nothing (three here: a step costs seconds on a large matrix, not milliseconds).
+      int struggle = 0;
+      const double T3 = sort_first ? 0.8 * T : T;
+    for (size_t bi = 0; bi < bands.size() && now_s() < T3; bi++) {
+        StrategyNode div = make_strategy(DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY, bands[bi][0], bands[bi][1], bands[bi][2], 0);
+        std::vector<uint64_t> cut = strips_of(sorted_len, bands[bi][0], bands[bi][1], bands[bi][2]);
+        if (cut.size() > 4 || cut.size() < 2) continue;
+        if (std::find(seen.begin(), seen.end(), cut) != seen.end()) continue;  // same strips as an earlier combination
+        seen.push_back(cut);
+        c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
+        BestGraph g;
+        double budget = (T - now_s()) / 2;
+        if (search_dense_strategy(c, in, {input, sort, div, compress}, budget, g) && g.gflops > best3.gflops) {
+          best3 = g;
+          struggle = 0;
+        } else if (best3.gflops > 0 && ++struggle >= 3) {
+          c.log("three row divisions in a row without an improvement: strategy 3 ends" + c.stamp());
+          break;
+        }
+      }
+      if (best3.gflops > 0) consider(best3, "strategy3");
+    }
+  };
+  if (sort_first) {
+    strategy3();
+    strategy1();
+    strategy2();
+  } else {
+    strategy1();
+    strategy2();
+    strategy3();
   }
   // strategies whose best graphs are within measurement noise of each other are measured again,
   // each over a region four times as long, and the faster one is kept
