@@ -61,6 +61,7 @@ MEASURED_TRAFFIC = {
     "e9afcd580f447551": 197734396,    # C3, tile kernel of the long strip + its finish (pin sort+div64|T1@1024|T2:slice=8192,group=65536@512)
     "dad308d7a3b7a127": 711696691,    # C4, tile kernel, column runs, row ownership, blocks of 3 rows (pin |T1:slice=16384,group=4092@1024,runs,own,blk3)
     "3b570d6d4c746c50": 803162829,    # C4, the same without row blocks (pin |T1:slice=16384,group=4096@1024,runs,own)
+    "4f3d4599ea632134": 701548339,    # C5, the same graph with the thread counts the search picks (tile @512, product-bin @1024)
     "b9791554820cbb6f": 688027956,    # C5, product-bin kernel, both passes (pin sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256)
 }
 
