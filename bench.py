@@ -324,7 +324,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (rows would shard across GPUs with x "
-              "replicated; see DESIGN.md).  Run with --gpus 1.", file=sys.stderr)
+              "replicated and no reduction).  Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if args.pin and not args.workload:
         print("bench.py: --pin needs --workload", file=sys.stderr)

@@ -1,4 +1,5 @@
-"""The reference-side binding that INTEGRATION.md documents for part_execute_code_builder (executor.hpp:12-17),
+"""The reference-side binding of part_execute_code_builder (executor.hpp:12-17): a body that keeps the reference's own
+signature and calls the C-ABI,
 compiled as a C++ program against include/alphasparse_amd.h (tests/integration/part_execute_wrapper.cc, built by
 alphasparse_amd/csrc/Makefile) and run on the GPU: repeat = 0 must take the reference's own launch count
 (executor.cc:247-255: 185.2e9 / padded elements, at least 2)."""
