@@ -48,9 +48,23 @@ def _bind(L):
     L.as_builder_time.argtypes = [vp, C.c_uint64, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.as_builder_algorithmic_bytes.restype = C.c_int64
     L.as_builder_algorithmic_bytes.argtypes = [vp]
+    L.as_builder_scratch_bytes.restype = C.c_int64
+    L.as_builder_scratch_bytes.argtypes = [vp, C.c_int64]
     L.as_hip_device_count.restype = C.c_int
     L.as_builder_spmv_device.argtypes = [vp, vp, vp]
     L.as_builder_spmv_device_no_alloc.argtypes = [vp, vp, vp]
+    L.as_builder_spmv_device_async.argtypes = [vp, vp, vp, vp]
+    L.as_builder_spmv_device_no_alloc_async.argtypes = [vp, vp, vp, vp]
+    L.as_builder_stream.restype = vp
+    L.as_builder_stream.argtypes = [vp]
+    L.as_hip_stream_create.argtypes = [C.POINTER(vp)]
+    L.as_hip_stream_destroy.argtypes = [vp]
+    L.as_hip_stream_sync.argtypes = [vp]
+    L.as_hip_graph_capture_begin.argtypes = [vp]
+    L.as_hip_graph_capture_end.argtypes = [vp, C.POINTER(vp)]
+    L.as_hip_graph_launch.argtypes = [vp, vp]
+    L.as_hip_graph_destroy.argtypes = [vp]
+    L.as_hip_mem_info.argtypes = [capi.u64p, capi.u64p]
     L.as_builder_clears_y.argtypes = [vp]
     L.as_builder_static_scratch_need.restype = C.c_int64
     L.as_builder_static_scratch_need.argtypes = [vp]
@@ -60,6 +74,108 @@ def _bind(L):
     L.as_hip_h2d.argtypes = [vp, vp, C.c_uint64]
     L.as_hip_d2h.argtypes = [vp, vp, C.c_uint64]
     _bound = True
+
+
+def device_facts(read_device=None, cu_num=0, lds_bytes=0):
+    """What the format builders assume about the GPU, as a dict (cu_num, lds_bytes, xcd_num, l2_bytes_per_xcd,
+    from_device).  read_device = a GPU number: ask that GPU first; cu_num / lds_bytes != 0: set them first."""
+    L = capi.lib()
+    L.as_device_facts.argtypes = [capi.u64p, capi.u64p, capi.u64p, capi.u64p, capi.intp]
+    L.as_device_facts_set.argtypes = [C.c_uint64, C.c_uint64]
+    L.as_device_facts_read.argtypes = [C.c_int]
+    if read_device is not None and L.as_device_facts_read(int(read_device)) != 0:
+        raise capi.AlphaSparseError(L.as_last_error().decode())
+    if (cu_num or lds_bytes) and L.as_device_facts_set(int(cu_num), int(lds_bytes)) != 0:
+        raise capi.AlphaSparseError(L.as_last_error().decode())
+    v = [C.c_uint64(0) for _ in range(4)]
+    f = C.c_int(0)
+    if L.as_device_facts(*[C.byref(a) for a in v], C.byref(f)) != 0:
+        raise capi.AlphaSparseError(L.as_last_error().decode())
+    return {"cu_num": v[0].value, "lds_bytes": v[1].value, "xcd_num": v[2].value, "l2_bytes_per_xcd": v[3].value,
+            "from_device": bool(f.value)}
+
+
+class DeviceArray:
+    """A caller-owned device buffer (as_hip_alloc) holding a numpy array's bytes: what a user of the C-ABI passes to
+    the *_device entry points."""
+
+    def __init__(self, host):
+        self._L = capi.lib()
+        _bind(self._L)
+        host = np.ascontiguousarray(host)
+        self.dtype, self.shape, self.nbytes = host.dtype, host.shape, host.nbytes
+        self.ptr = C.c_void_p()
+        if self._L.as_hip_alloc(C.byref(self.ptr), max(1, self.nbytes)) != 0:
+            raise capi.AlphaSparseError(self._L.as_hip_last_error().decode())
+        self.set(host)
+
+    def set(self, host):
+        host = np.ascontiguousarray(host, dtype=self.dtype)
+        assert host.nbytes == self.nbytes
+        if self._L.as_hip_h2d(self.ptr, host.ctypes.data_as(C.c_void_p), self.nbytes) != 0:
+            raise capi.AlphaSparseError(self._L.as_hip_last_error().decode())
+
+    def get(self):
+        out = np.empty(self.shape, self.dtype)
+        if self._L.as_hip_d2h(out.ctypes.data_as(C.c_void_p), self.ptr, self.nbytes) != 0:
+            raise capi.AlphaSparseError(self._L.as_hip_last_error().decode())
+        return out
+
+    def free(self):
+        if self.ptr:
+            self._L.as_hip_free(self.ptr)
+            self.ptr = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Stream:
+    """A HIP stream of the caller (default priority), with the capture and replay calls of the thin HIP layer."""
+
+    def __init__(self):
+        self._L = capi.lib()
+        _bind(self._L)
+        self.ptr = C.c_void_p()
+        self._hip(self._L.as_hip_stream_create(C.byref(self.ptr)))
+
+    def _hip(self, status):
+        if status != 0:
+            raise capi.AlphaSparseError(self._L.as_hip_last_error().decode())
+
+    def sync(self):
+        self._hip(self._L.as_hip_stream_sync(self.ptr))
+
+    def capture_begin(self):
+        self._hip(self._L.as_hip_graph_capture_begin(self.ptr))
+
+    def capture_end(self):
+        g = C.c_void_p()
+        self._hip(self._L.as_hip_graph_capture_end(self.ptr, C.byref(g)))
+        return g
+
+    def graph_launch(self, graph_exec):
+        self._hip(self._L.as_hip_graph_launch(graph_exec, self.ptr))
+
+    def graph_destroy(self, graph_exec):
+        self._hip(self._L.as_hip_graph_destroy(graph_exec))
+
+    def destroy(self):
+        if self.ptr:
+            self._L.as_hip_stream_destroy(self.ptr)
+            self.ptr = C.c_void_p()
+
+
+def device_memory_free_bytes():
+    L = capi.lib()
+    _bind(L)
+    f, t = C.c_uint64(0), C.c_uint64(0)
+    if L.as_hip_mem_info(C.byref(f), C.byref(t)) != 0:
+        raise capi.AlphaSparseError(L.as_hip_last_error().decode())
+    return f.value
 
 
 def kernel_cache_stats():
@@ -213,6 +329,18 @@ class Builder:
         self._chk(self._L.as_builder_spmv(self._h, x.ctypes.data_as(C.c_void_p), y.ctypes.data_as(C.c_void_p)))
         return y
 
+    def spmv_device_async(self, x_dev, y_dev, stream=None, no_alloc=False):
+        """Enqueue y = A x on the caller's stream (a Stream, or None for the builder's own stream) and return:
+        as_builder_spmv_device_async / as_builder_spmv_device_no_alloc_async on DeviceArray buffers."""
+        call = self._L.as_builder_spmv_device_no_alloc_async if no_alloc else self._L.as_builder_spmv_device_async
+        s = stream.ptr if stream is not None else self._L.as_builder_stream(self._h)
+        self._chk(call(self._h, x_dev.ptr, y_dev.ptr, s))
+
+    def sync(self):
+        """Wait for the builder's own stream."""
+        if self._L.as_hip_stream_sync(self._L.as_builder_stream(self._h)) != 0:
+            raise capi.AlphaSparseError(self._L.as_hip_last_error().decode())
+
     def spmv_device(self, x, y_before=None, no_alloc=False):
         """y = A x on device buffers of the caller (as_builder_spmv_device, or as_builder_spmv_device_no_alloc): y
         holds `y_before` (a scalar or an array; default NaN) when the call starts, so a row that no kernel writes,
@@ -284,6 +412,10 @@ class Builder:
 
     def algorithmic_bytes(self):
         return int(self._chk(self._L.as_builder_algorithmic_bytes(self._h)))
+
+    def scratch_bytes(self, sub=-1):
+        """Bytes of the kernels' scratch arrays (products, row sums) of one sub-matrix, or of all."""
+        return int(self._chk(self._L.as_builder_scratch_bytes(self._h, sub)))
 
     def close(self):
         if self._h:

@@ -1,5 +1,6 @@
 // extern "C" surface declared in include/alphasparse_amd.h (matrix / graph part).
 #include "capi_internal.hpp"
+#include "device_facts.hpp"
 
 #include <cstring>
 
@@ -9,6 +10,33 @@ extern "C" {
 
 const char *as_last_error(void) { return g_as_last_error.c_str(); }
 const char *as_version(void) { return "alphasparse_amd 0.1 (gfx950)"; }
+
+int as_device_facts(uint64_t *cu_num, uint64_t *lds_bytes, uint64_t *xcd_num, uint64_t *l2_bytes_per_xcd, int *from_device) {
+  AS_API_BEGIN
+  const asx::DeviceFacts &f = asx::device_facts();
+  if (cu_num) *cu_num = f.cu_num;
+  if (lds_bytes) *lds_bytes = f.lds_bytes;
+  if (xcd_num) *xcd_num = asx::kXcdNum;
+  if (l2_bytes_per_xcd) *l2_bytes_per_xcd = asx::kL2BytesPerXcd;
+  if (from_device) *from_device = f.from_device ? 1 : 0;
+  return 0;
+  AS_API_END(-1)
+}
+
+int as_device_facts_read(int device) {
+  AS_API_BEGIN
+  asx::read_device_facts(device);
+  return 0;
+  AS_API_END(-1)
+}
+
+int as_device_facts_set(uint64_t cu_num, uint64_t lds_bytes) {
+  AS_API_BEGIN
+  AS_CHECK(lds_bytes == 0 || lds_bytes >= 65536, "at least 64 KB of LDS per workgroup");
+  asx::set_device_facts(cu_num, lds_bytes);
+  return 0;
+  AS_API_END(-1)
+}
 
 as_matrix *as_matrix_from_coo(uint64_t rows, uint64_t cols, uint64_t nnz, const uint64_t *row, const uint64_t *col,
                               const double *val, int val_dtype, int wave) {
@@ -242,8 +270,10 @@ int as_execute_node(as_matrix *m, int node_type, int64_t sub, const long *scalar
     case asx::DENSE_ROW_COARSE_SORT:
       n.bin_row_nnz_low_bound.assign(list, list + n_list);
       break;
-    case asx::DENSE_ROW_DIV:
+    case asx::DENSE_ROW_DIV:  // scalars (optional): {dense_sub_block_id [, height of equal strips when the list is empty]}
       n.row_div_position.assign(list, list + n_list);
+      if (n_scalars >= 1) n.dense_sub_block_id = (uint64_t)scalars[0];
+      if (n_scalars >= 2) n.fixed_row_block_size = scalars[1];
       break;
     case asx::DENSE_FINE_SORT:
       n.first_row_of_each_sort_band.assign(list, list + n_list);
@@ -252,8 +282,9 @@ int as_execute_node(as_matrix *m, int node_type, int64_t sub, const long *scalar
       n.sort_block_index_arr.assign(list, list + n_list);
       break;
     case asx::DENSE_FIXED_COL_DIV:
-      AS_CHECK(n_scalars >= 1, "need {fixed_col_block_size}");
+      AS_CHECK(n_scalars >= 1, "need {fixed_col_block_size [, dense_sub_block_id]}");
       n.fixed_col_block_size = scalars[0];
+      if (n_scalars >= 2) n.dense_sub_block_id = (uint64_t)scalars[1];
       break;
     default:
       break;

@@ -221,6 +221,24 @@ int as_builder_spmv_device_no_alloc(as_builder *b, const void *x_dev, void *y_de
   AS_API_END(-1)
 }
 
+int as_builder_spmv_device_async(as_builder *b, const void *x_dev, void *y_dev, void *stream) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b && x_dev && y_dev, "null argument");
+  asx::launch_spmv(*b->b, x_dev, y_dev, stream);
+  return 0;
+  AS_API_END(-1)
+}
+
+int as_builder_spmv_device_no_alloc_async(as_builder *b, const void *x_dev, void *y_dev, void *stream) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b && x_dev && y_dev, "null argument");
+  asx::launch_spmv_no_alloc(*b->b, x_dev, y_dev, stream);
+  return 0;
+  AS_API_END(-1)
+}
+
+void *as_builder_stream(as_builder *b) { return b && b->b ? b->b->main_stream : nullptr; }
+
 int64_t as_builder_static_scratch_need(as_builder *b) {
   AS_API_BEGIN
   AS_CHECK(b && b->b, "null builder");
@@ -321,6 +339,16 @@ int as_builder_time(as_builder *b, uint64_t reps, int sync_each_launch, float *t
   AS_CHECK(b && b->b && time_ms && gflops, "null argument");
   asx::time_spmv(*b->b, reps, sync_each_launch != 0, *time_ms, *gflops);
   return 0;
+  AS_API_END(-1)
+}
+
+int64_t as_builder_scratch_bytes(as_builder *b, int64_t sub) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b, "null builder");
+  uint64_t bytes = 0;
+  for (size_t s = 0; s < b->b->subs.size(); s++)
+    if (b->b->subs[s].tpl && (sub < 0 || (int64_t)s == sub)) bytes += b->b->subs[s].tpl->scratch_bytes;
+  return (int64_t)bytes;
   AS_API_END(-1)
 }
 
@@ -534,6 +562,35 @@ void as_search_free(as_search_result *r) { delete r; }
 const char *as_search_report(const as_search_result *r) { return r ? r->report.c_str() : ""; }
 const char *as_search_log(const as_search_result *r) { return r ? r->r.log.c_str() : ""; }
 
+int64_t as_search_best_graph(const as_search_result *r, long *desc, uint64_t cap) {
+  AS_API_BEGIN
+  AS_CHECK(r, "null argument");
+  std::vector<long> d;
+  auto nodes = [&](const std::vector<asx::StrategyNode> &v) {
+    d.push_back((long)v.size());
+    for (const asx::StrategyNode &n : v) {
+      d.push_back((long)n.strategy);
+      if (n.strategy == asx::DENSE_BEGIN_MEMORY_CACHE_INPUT_FILE_DIRECT_PARAM_STRATEGY) {
+        d.push_back((long)n.in_nnz); d.push_back((long)n.in_val_dtype);
+        d.push_back((long)n.in_col_index_max); d.push_back((long)n.in_row_index_max);
+      } else {
+        for (int i = 0; i < 4; i++) d.push_back(n.p[i]);
+      }
+    }
+  };
+  nodes(r->r.best.dense);
+  d.push_back((long)r->r.best.subs.size());
+  for (const asx::SubGraph &sub : r->r.best.subs) {
+    nodes(sub.nodes);
+    d.push_back((long)sub.tpl.type); d.push_back(sub.tpl.tblock_num);
+    d.push_back(sub.tpl.thread_num_in_block); d.push_back(sub.tpl.thread_num_of_row_reduce);
+  }
+  if (desc)
+    for (size_t i = 0; i < d.size() && i < cap; i++) desc[i] = d[i];
+  return (int64_t)d.size();
+  AS_API_END(-1)
+}
+
 int as_search_stats(const as_search_result *r, double out[8]) {
   AS_API_BEGIN
   AS_CHECK(r && out, "null argument");
@@ -637,6 +694,45 @@ extern "C" int64_t as_strategy_report(int strategy, const long p[4], char *out, 
   AS_CHECK(p, "bad argument");
   asx::StrategyNode n = asx::make_strategy((asx::ParamStrategy)strategy, p[0], p[1], p[2], p[3]);
   return put_text(asx::convert_stategy_node_to_string(n), out, cap);
+  AS_API_END(-1)
+}
+
+extern "C" int64_t as_graph_report(const long *desc, int64_t n_desc, int with_frame, float gflops, float time_ms, char *out,
+                                   uint64_t cap) {
+  AS_API_BEGIN
+  AS_CHECK(desc && n_desc >= 2, "bad argument");
+  int64_t at = 0;
+  auto need = [&](int64_t more) { AS_CHECK(at + more <= n_desc, "the description of the graph ends early"); };
+  auto node = [&]() {
+    need(5);
+    asx::StrategyNode n = asx::make_strategy((asx::ParamStrategy)desc[at], desc[at + 1], desc[at + 2], desc[at + 3], desc[at + 4]);
+    if (n.strategy == asx::DENSE_BEGIN_MEMORY_CACHE_INPUT_FILE_DIRECT_PARAM_STRATEGY) {
+      n.in_nnz = (uint64_t)desc[at + 1];
+      n.in_val_dtype = (asx::DType)desc[at + 2];
+      n.in_col_index_max = (uint64_t)desc[at + 3];
+      n.in_row_index_max = (uint64_t)desc[at + 4];
+    }
+    at += 5;
+    return n;
+  };
+  asx::BestGraph g;
+  need(1);
+  for (long i = 0, n = desc[at++]; i < n; i++) g.dense.push_back(node());
+  need(1);
+  for (long s = 0, n_sub = desc[at++]; s < n_sub; s++) {
+    asx::SubGraph sub;
+    need(1);
+    for (long i = 0, n = desc[at++]; i < n; i++) sub.nodes.push_back(node());
+    need(4);
+    sub.tpl.type = (asx::TemplateType)desc[at];
+    sub.tpl.tblock_num = desc[at + 1];
+    sub.tpl.thread_num_in_block = desc[at + 2];
+    sub.tpl.thread_num_of_row_reduce = desc[at + 3];
+    at += 4;
+    g.subs.push_back(sub);
+  }
+  AS_CHECK(at == n_desc, "the description of the graph is longer than the graph");
+  return put_text(with_frame ? asx::convert_search_result_to_string(gflops, time_ms, g) : asx::convert_graph_to_string(g), out, cap);
   AS_API_END(-1)
 }
 

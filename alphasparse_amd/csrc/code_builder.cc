@@ -4,6 +4,7 @@
 
 #include <cstring>
 
+#include "device_facts.hpp"
 #include "hip_layer.h"
 
 namespace asx {
@@ -174,6 +175,29 @@ bool set_row_blocks(Builder &b, uint64_t sub, uint64_t rows_per_block) {
   return true;
 }
 
+bool add_tile_template_variant_to_builder(Builder &b, uint64_t sub, bool column_runs_if_shorter, bool own_rows, uint64_t row_block) {
+  AS_CHECK(b.matrix != nullptr && sub < b.subs.size(), "sub-matrix id out of range");
+  // column runs where set_column_runs would take them: the stream must get at least 2 % shorter, lane-closing
+  // padding included; counted in one pass before anything is built
+  const double vs = (double)dtype_size(b.matrix->val_dtype);
+  const CompressedBlock &cb = *b.matrix->items[sub].cb;
+  const double plain = (double)cb.read_index[0]->index_arr.v.size() * (vs + 2.5);
+  const bool runs = column_runs_if_shorter && (double)tile_column_run_stream_estimate(*b.matrix, sub) * (vs + 1.625) <= 0.98 * plain;
+  std::unique_ptr<Template> t = init_tile_template_variant(*b.matrix, sub, runs, own_rows, row_block);
+  if (!t) return false;
+  try_all_compress(*t);
+  t->y_needs_clear = template_needs_cleared_y(*t, *b.matrix, sub);
+  set_default_launch(*t);
+  if (b.subs[sub].uploaded) {
+    as_hip_device_sync();
+    free_sub_arrays(b.subs[sub]);
+    b.subs[sub].uploaded = false;
+  }
+  b.subs[sub].tpl = std::move(t);
+  invalidate(b);
+  return true;
+}
+
 bool set_column_runs(Builder &b, uint64_t sub) {
   AS_CHECK(b.matrix != nullptr && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template");
   Template &old = *b.subs[sub].tpl;
@@ -306,6 +330,8 @@ static void ensure_module(Builder &b) {
   HIPL(as_hip_get_kernel(b.module, "as_zero_words", &b.zero_fn));
   for (auto &k : b.subs) {
     if (!k.tpl) continue;
+    k.fn = k.finish_fn = nullptr;
+    if (k.tpl->type == EMPTY_TEMPLATE) continue;  // no kernel
     std::string name = "spmv_" + std::to_string(k.tpl->sub);
     HIPL(as_hip_get_kernel(b.module, name.c_str(), &k.fn));
     k.finish_fn = nullptr;
@@ -317,6 +343,7 @@ static void ensure_module(Builder &b) {
 void load_and_upload(Builder &b, int device) {
   if (!b.device_ready) {
     HIPL(as_hip_init(device));
+    read_device_facts(device);
     HIPL(as_hip_stream_create(&b.main_stream));
     HIPL(as_hip_event_create(&b.start_ev));
     HIPL(as_hip_event_create(&b.t0));
@@ -327,7 +354,11 @@ void load_and_upload(Builder &b, int device) {
     HIPL(as_hip_alloc(&b.y.ptr, b.rows * vs));
     b.y.bytes = b.rows * vs;
     // the static scratch array of this GPU, for the entry point that allocates nothing: looked up here, once
-    HIPL(as_hip_static_scratch(device, &b.static_scratch, &b.static_scratch_bytes));
+    // (a failed lookup only disables that entry point, which then says so)
+    if (as_hip_static_scratch(device, &b.static_scratch, &b.static_scratch_bytes) != 0) {
+      b.static_scratch = nullptr;
+      b.static_scratch_bytes = 0;
+    }
     b.device_ready = true;
   }
   ensure_module(b);
@@ -348,12 +379,12 @@ void load_and_upload(Builder &b, int device) {
 
 // Launches the kernels of every active sub-matrix.  static_scratch != nullptr: the kernels' scratch arrays are
 // 256-byte aligned pieces of that memory (in sub-matrix order) instead of the builder's own allocations.
-static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned char *static_scratch = nullptr) {
+static void launch_kernels(Builder &b, void *stream, const void *x_dev, void *y_dev, unsigned char *static_scratch = nullptr) {
   size_t active = 0;
   auto skipped = [&](const SubKernel &k) { return !k.tpl || (b.only_sub >= 0 && &k != &b.subs[(size_t)b.only_sub]); };
   for (auto &k : b.subs) active += !skipped(k);
   bool multi = active > 1 && !b.serial_launch;
-  if (multi) HIPL(as_hip_event_record(b.start_ev, b.main_stream));
+  if (multi) HIPL(as_hip_event_record(b.start_ev, stream));
   uint64_t scratch_offset = 0;
   const SubKernel *before = nullptr;  // the sub-matrix with a template in front of the current one
   void *scratch_before = nullptr;
@@ -371,6 +402,7 @@ static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned 
       scratch_before = scratch_ptr;
     }
     if (skipped(k)) continue;
+    if (k.tpl->type == EMPTY_TEMPLATE) continue;  // nothing to launch: its rows of y are the clear's
     AS_CHECK(k.uploaded && k.fn, "a template was changed after upload: call upload again");
     // kernel arguments: passed metadata arrays, val, col, x, y, scratch -- a fixed-size list, nothing allocated
     void *ptrs[kMaxKernelArgs], *args[kMaxKernelArgs];
@@ -413,7 +445,7 @@ static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned 
           finish_is_carried = b.subs[j].tpl->carried == k.tpl.get();
           break;
         }
-    void *s = multi ? k.stream : b.main_stream;
+    void *s = multi ? k.stream : stream;
     if (multi) HIPL(as_hip_stream_wait_event(s, b.start_ev));
     if (b.only_pass != 2)
       HIPL(as_hip_launch(k.fn, (unsigned)(k.tpl->tblock_num + k.tpl->carried_blocks), (unsigned)k.tpl->thread_num_in_block,
@@ -425,26 +457,26 @@ static void launch_kernels(Builder &b, const void *x_dev, void *y_dev, unsigned 
     }
     if (multi) {
       HIPL(as_hip_event_record(k.done, s));
-      HIPL(as_hip_stream_wait_event(b.main_stream, k.done));
+      HIPL(as_hip_stream_wait_event(stream, k.done));
     }
   }
 }
 
-static void zero_words(Builder &b, void *p, unsigned long long words) {
+static void zero_words(Builder &b, void *stream, void *p, unsigned long long words) {
   void *args[] = {&p, &words};
   unsigned grid = (unsigned)std::min<unsigned long long>(4096, (words + 255) / 256);
-  HIPL(as_hip_launch(b.zero_fn, std::max(1u, grid), 256, 0, b.main_stream, args));
+  HIPL(as_hip_launch(b.zero_fn, std::max(1u, grid), 256, 0, stream, args));
 }
 
-static void zero_y(Builder &b, void *y_dev) {
-  zero_words(b, y_dev, (unsigned long long)b.rows * dtype_size(b.val_dtype) / 4);
+static void zero_y(Builder &b, void *stream, void *y_dev) {
+  zero_words(b, stream, y_dev, (unsigned long long)b.rows * dtype_size(b.val_dtype) / 4);
 }
 
 void clear_scratch(Builder &b, uint64_t sub) {
   AS_CHECK(b.device_ready && sub < b.subs.size() && b.subs[sub].tpl, "sub-matrix has no template on the device");
   SubKernel &k = b.subs[sub];
   if (!k.tpl->scratch_bytes || !k.scratch.ptr) return;
-  zero_words(b, k.scratch.ptr, (k.tpl->scratch_bytes + 3) / 4);
+  zero_words(b, b.main_stream, k.scratch.ptr, (k.tpl->scratch_bytes + 3) / 4);
   HIPL(as_hip_stream_sync(b.main_stream));
 }
 
@@ -465,13 +497,14 @@ static void check_launch_shapes(const Builder &b) {
   }
 }
 
-void launch_spmv(Builder &b, const void *x_dev, void *y_dev) {
+void launch_spmv(Builder &b, const void *x_dev, void *y_dev, void *stream) {
   AS_CHECK(b.device_ready, "builder is not on the device");
   ensure_module(b);
   check_launch_shapes(b);
-  if (y_needs_clear(b)) zero_y(b, y_dev);
-  launch_kernels(b, x_dev, y_dev);
+  if (y_needs_clear(b)) zero_y(b, stream, y_dev);
+  launch_kernels(b, stream, x_dev, y_dev);
 }
+void launch_spmv(Builder &b, const void *x_dev, void *y_dev) { launch_spmv(b, x_dev, y_dev, b.main_stream); }
 
 uint64_t static_scratch_need(const Builder &b) {
   uint64_t need = 0;
@@ -480,26 +513,27 @@ uint64_t static_scratch_need(const Builder &b) {
   return need;
 }
 
-void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev) {
+void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev) { launch_spmv_no_alloc(b, x_dev, y_dev, b.main_stream); }
+void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev, void *stream) {
   AS_CHECK(b.device_ready && b.module && !b.module_stale, "builder is not on the device: call upload first (this entry point loads nothing)");
   for (auto &k : b.subs) AS_CHECK(!k.tpl || k.uploaded, "a template was changed after upload: call upload again");
   check_launch_shapes(b);
   const uint64_t need = static_scratch_need(b);
+  AS_CHECK(need == 0 || b.static_scratch, "no static scratch array on this device (its address could not be looked up at upload): use as_builder_spmv_device");
   AS_CHECK(need <= b.static_scratch_bytes,
            "the kernels of this graph need " + std::to_string(need) + " bytes of scratch, the static scratch array holds " +
                std::to_string(b.static_scratch_bytes) + ": use as_builder_spmv_device");
-  AS_CHECK(need == 0 || b.static_scratch, "no static scratch array on this device");
   unsigned char *base = (unsigned char *)b.static_scratch;
   // Every call on this GPU shares the array, which holds what the last call left: the pieces whose kernels add
   // into them are cleared by the fill kernel (no memset node, so the sequence can be captured)
   uint64_t offset = 0;
   for (auto &k : b.subs) {
     if (!k.tpl || !k.tpl->scratch_bytes) continue;
-    if (k.tpl->scratch_starts_zero) zero_words(b, base + offset, (k.tpl->scratch_bytes + 3) / 4);
+    if (k.tpl->scratch_starts_zero) zero_words(b, stream, base + offset, (k.tpl->scratch_bytes + 3) / 4);
     offset += (k.tpl->scratch_bytes + 255) / 256 * 256;
   }
-  if (y_needs_clear(b)) zero_y(b, y_dev);
-  launch_kernels(b, x_dev, y_dev, base ? base : nullptr);
+  if (y_needs_clear(b)) zero_y(b, stream, y_dev);
+  launch_kernels(b, stream, x_dev, y_dev, base ? base : nullptr);
 }
 
 void spmv_host(Builder &b, const void *x_host, void *y_host) {
@@ -518,13 +552,13 @@ void time_spmv(Builder &b, uint64_t reps, bool sync_each, float &time_ms, float 
   // it.  Measurements of one sub-matrix's kernels alone (only_sub) are kernel times: y is cleared once, before.
   const bool clear_each = b.only_sub < 0 && y_needs_clear(b);
   if (b.only_sub >= 0) {
-    zero_y(b, b.y.ptr);
+    zero_y(b, b.main_stream, b.y.ptr);
     HIPL(as_hip_stream_sync(b.main_stream));
   }
   HIPL(as_hip_event_record(b.t0, b.main_stream));
   for (uint64_t r = 0; r < reps; r++) {
-    if (clear_each) zero_y(b, b.y.ptr);
-    launch_kernels(b, b.x.ptr, b.y.ptr);
+    if (clear_each) zero_y(b, b.main_stream, b.y.ptr);
+    launch_kernels(b, b.main_stream, b.x.ptr, b.y.ptr);
     if (sync_each) HIPL(as_hip_stream_sync(b.main_stream));
   }
   HIPL(as_hip_event_record(b.t1, b.main_stream));

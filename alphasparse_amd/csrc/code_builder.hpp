@@ -61,6 +61,11 @@ bool compress_template_in_builder(Builder &b, uint64_t sub);                    
 bool set_relative_columns(Builder &b, uint64_t sub);
 // make_columns_diagonal on the template of one sub-matrix; same rules
 bool set_diagonal_columns(Builder &b, uint64_t sub);
+// The tile template of a sub-matrix built at once in a combination of its forms (row ownership, blocks of rows as
+// pieces, column runs where they make the element stream at least 2 % shorter): what the search measures first on a
+// banded matrix whose rows come in blocks, instead of walking there one form at a time.  false (builder unchanged)
+// where the combination does not apply.
+bool add_tile_template_variant_to_builder(Builder &b, uint64_t sub, bool column_runs_if_shorter, bool own_rows, uint64_t row_block);
 // Rebuilds the tile template of a sub-matrix in its column-run form (init_tile_template_with_column_runs) and
 // keeps it when the element stream gets shorter by at least 2 %; false (template unchanged) otherwise, or when
 // the sub-matrix has another template.  The launch setting is kept.
@@ -91,11 +96,14 @@ void clear_scratch(Builder &b, uint64_t sub);
 int64_t assign_finish_carriers(const Builder &b, uint64_t sub = ~0ull);
 // y = A x on device buffers already holding x; y is cleared first where y_needs_clear says so.
 void launch_spmv(Builder &b, const void *x_dev, void *y_dev);
+// the same on a stream of the caller (a hipStream_t; nullptr = the default stream): enqueues and returns
+void launch_spmv(Builder &b, const void *x_dev, void *y_dev, void *stream);
 // The same SpMV for callers that must not allocate device memory: nothing is compiled, loaded or allocated
 // (the builder must be uploaded), and the kernels' scratch arrays are pieces of the library's static scratch
 // array on this GPU instead of the builder's own.  Fails when the graph needs more scratch than the array holds.
 // Calls that overlap on one GPU share the array and race.
 void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev);
+void launch_spmv_no_alloc(Builder &b, const void *x_dev, void *y_dev, void *stream);
 uint64_t static_scratch_need(const Builder &b);  // bytes of the static array the graph's kernels would use
 void spmv_host(Builder &b, const void *x_host, void *y_host);
 // Timing: `reps` launches of all kernels.  sync_each_launch reproduces the

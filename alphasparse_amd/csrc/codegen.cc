@@ -1,4 +1,5 @@
 // Source emission helpers shared by the kernel templates.
+#include "device_facts.hpp"
 #include "templates.hpp"
 
 namespace asx {
@@ -9,7 +10,7 @@ std::string y_row_type_name(const Template &) { return "unsigned int"; }
 // Everything the generated kernels rely on.  Written for gfx950 only: 64-lane
 // wavefronts, DPP row operations, hardware floating-point atomics.
 std::string kernel_module_preamble() {
-  return R"SRC(
+  return "#define AS_XCD_NUM " + std::to_string(kXcdNum) + "u\n" + R"SRC(
 #define AS_WAVE 64
 typedef unsigned int as_u32;
 typedef unsigned long long as_u64;
@@ -26,7 +27,7 @@ __device__ __forceinline__ void as_atomic_add(double *p, double v) { unsafeAtomi
 // here instead of blockIdx.x: every XCD then works on a contiguous eighth of the blocks, and a line of x
 // that two neighbouring blocks need is fetched into one L2, not two.  A permutation of [0, gridDim.x).
 __device__ __forceinline__ unsigned int as_xcd_block_index(unsigned int b, unsigned int n) {
-  return b < (n & ~7u) ? (b & 7u) * (n >> 3) + (b >> 3) : b;
+  return b < n / AS_XCD_NUM * AS_XCD_NUM ? (b % AS_XCD_NUM) * (n / AS_XCD_NUM) + b / AS_XCD_NUM : b;
 }
 __device__ __forceinline__ unsigned int as_xcd_block_index() { return as_xcd_block_index(blockIdx.x, gridDim.x); }
 

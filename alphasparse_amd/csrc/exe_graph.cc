@@ -35,15 +35,25 @@ void execute_dense_node(Matrix &m, const ExeNode &node) {
     case DENSE_FINE_SORT:  // op_manager API upstream (no node executor there)
       total_dense_block_sort(m, node.first_row_of_each_sort_band);
       return;
-    case DENSE_ROW_DIV:
-      if (node.row_div_position.size() <= 2) return;  // a single strip is a no-op
-      AS_CHECK(m.items.empty() && node.dense_sub_block_id == 0, "further division of a sub-block is not supported");
-      var_len_row_div(m, node.row_div_position);
+    case DENSE_ROW_DIV:  // exe_graph.cc:1574-1613: the whole matrix first, a sub-block of the table afterwards
+      if (m.items.empty()) {
+        AS_CHECK(node.dense_sub_block_id == 0, "the matrix has no sub-blocks yet");
+        if (node.row_div_position.size() <= 2) return;  // a single strip is a no-op
+        var_len_row_div(m, node.row_div_position);
+      } else if (node.row_div_position.empty() && node.fixed_row_block_size > 0) {
+        fixed_len_row_div(m, (uint64_t)node.fixed_row_block_size, node.dense_sub_block_id);
+      } else {
+        var_len_row_div(m, node.row_div_position, node.dense_sub_block_id);
+      }
       return;
-    case DENSE_FIXED_COL_DIV:  // exe_graph.cc:1615
+    case DENSE_FIXED_COL_DIV:  // exe_graph.cc:1615-1640
       AS_CHECK(node.fixed_col_block_size > 0, "band width must be positive");
-      AS_CHECK(m.items.empty() && node.dense_sub_block_id == 0, "further division of a sub-block is not supported");
-      fixed_len_col_div(m, (uint64_t)node.fixed_col_block_size);
+      if (m.items.empty()) {
+        AS_CHECK(node.dense_sub_block_id == 0, "the matrix has no sub-blocks yet");
+        fixed_len_col_div(m, (uint64_t)node.fixed_col_block_size);
+      } else {
+        fixed_len_col_div(m, (uint64_t)node.fixed_col_block_size, node.dense_sub_block_id);
+      }
       return;
     case COMPRESS:
       compress_dense_view(m);
@@ -200,10 +210,19 @@ void execute_param_strategy_node_of_dense_matrix(StrategyNode &n, Matrix &m) {
     }
     case DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY: {  // :534-592
       AS_CHECK(n.p[2] > 0 && n.p[0] > 0, "expansion rate and lowest bound must be positive");
-      AS_CHECK(m.items.empty() && n.p[3] == 0, "further division of a sub-block is not supported");
       n.node.dense_sub_block_id = (uint64_t)n.p[3];
-      n.node.row_div_position = row_div_position_acc_to_exponential_increase_row_nnz_range(
-          get_nnz_of_each_row(m), (uint64_t)n.p[0], (uint64_t)n.p[1], (uint64_t)n.p[2]);
+      if (m.items.empty()) {
+        AS_CHECK(n.p[3] == 0, "the matrix has no sub-blocks yet");
+        n.node.row_div_position = row_div_position_acc_to_exponential_increase_row_nnz_range(
+            get_nnz_of_each_row(m), (uint64_t)n.p[0], (uint64_t)n.p[1], (uint64_t)n.p[2]);
+      } else {
+        // the bands of row length inside one sub-block (rows relative to its first row)
+        AS_CHECK((uint64_t)n.p[3] < m.items.size(), "sub-matrix id out of range");
+        const DenseItem &it = m.items[(size_t)n.p[3]];
+        std::vector<uint64_t> len(it.max_row - it.min_row + 1, 0);
+        for (uint64_t k = it.begin_coo; k <= it.end_coo; k++) len[m.coo_row[k] - it.min_row]++;
+        n.node.row_div_position = row_div_position_acc_to_exponential_increase_row_nnz_range(len, (uint64_t)n.p[0], (uint64_t)n.p[1], (uint64_t)n.p[2]);
+      }
       return;
     }
     default:

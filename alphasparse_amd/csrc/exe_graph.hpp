@@ -31,8 +31,13 @@ struct ExeNode {
   std::vector<uint64_t> first_row_of_each_sort_band;         // DENSE_FINE_SORT (empty: one band)
   std::vector<uint64_t> sort_block_index_arr;                // COMPRESSED_BLOCK_SORT (empty: every BLB)
   std::vector<uint64_t> row_div_position;                    // DENSE_ROW_DIV
+  // DENSE_ROW_DIV, DENSE_FIXED_COL_DIV: the sub-block of an already divided matrix that is cut (exe_graph.hpp
+  // exe_dense_row_div_param_t / exe_dense_fixed_col_div_param_t); 0 for the first division of the matrix
   uint64_t dense_sub_block_id = 0;
   long fixed_col_block_size = 0;                             // DENSE_FIXED_COL_DIV
+  // DENSE_ROW_DIV of a sub-block into strips of equal height (upstream fixed_len_row_div, op_manager.cc:127, an
+  // operator without a node of its own): used when row_div_position is empty
+  long fixed_row_block_size = 0;
   // COMPRESSED_TBLOCK_LEVEL_COL_DIV into 2-D tiles (row_group != 0): slice width, group height, BLB size
   uint64_t col_slice = 0, row_group = 0, block_nnz = 0;
   void reset_param();

@@ -213,6 +213,38 @@ int as_hip_event_elapsed_ms(void *start, void *stop, float *ms) {
   return 0;
 }
 // make `stream` wait for `ev`
+// Stream capture into a graph, for callers that replay a fixed sequence of launches (and for the test that the
+// enqueue-only SpMV calls can be captured).  Capture mode "thread local": only this thread's calls are checked.
+int as_hip_graph_capture_begin(void *stream) {
+  HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return 0;
+}
+int as_hip_graph_capture_end(void *stream, void **graph_exec) {
+  hipGraph_t g = nullptr;
+  HIP_TRY(hipStreamEndCapture((hipStream_t)stream, &g));
+  hipGraphExec_t e = nullptr;
+  hipError_t r = hipGraphInstantiate(&e, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (r != hipSuccess) return fail("hipGraphInstantiate", hipGetErrorString(r));
+  *graph_exec = e;
+  return 0;
+}
+int as_hip_graph_launch(void *graph_exec, void *stream) {
+  HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+  return 0;
+}
+int as_hip_graph_destroy(void *graph_exec) {
+  HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+  return 0;
+}
+int as_hip_mem_info(uint64_t *free_bytes, uint64_t *total_bytes) {
+  size_t f = 0, t = 0;
+  HIP_TRY(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return 0;
+}
+
 int as_hip_stream_wait_event(void *stream, void *ev) {
   HIP_TRY(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)ev, 0));
   return 0;

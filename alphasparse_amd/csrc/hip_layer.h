@@ -33,6 +33,11 @@ int as_hip_event_record(void *ev, void *stream);
 int as_hip_event_sync(void *ev);
 int as_hip_event_elapsed_ms(void *start, void *stop, float *ms);
 int as_hip_stream_wait_event(void *stream, void *ev);
+int as_hip_graph_capture_begin(void *stream);
+int as_hip_graph_capture_end(void *stream, void **graph_exec);
+int as_hip_graph_launch(void *graph_exec, void *stream);
+int as_hip_graph_destroy(void *graph_exec);
+int as_hip_mem_info(uint64_t *free_bytes, uint64_t *total_bytes);
 int as_hip_launch(void *fn, unsigned grid, unsigned block, unsigned lds_bytes, void *stream, void **args);
 #ifdef __cplusplus
 }

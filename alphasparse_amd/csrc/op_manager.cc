@@ -312,6 +312,90 @@ void fixed_len_row_div(Matrix &m, uint64_t len) {
   var_len_row_div(m, pos);
 }
 
+// Division of an EXISTING sub-block.  Upstream: fixed_len_row_div and fixed_len_col_div with sub_block != NULL
+// (op_manager.cc:243-365, 808-965); its var_len_row_div stops there ("further div is not support", :520), the
+// node DENSE_ROW_DIV passes a sub-block to it all the same (exe_graph.cc:1611), so the intent is plain: positions
+// relative to the sub-block's first row.  As upstream, the parent leaves the table and its parts are appended at
+// the end of it, in order; a part without elements is dropped.
+void var_len_row_div(Matrix &m, const std::vector<uint64_t> &pos, uint64_t sub) {
+  AS_CHECK(!m.is_compressed, "matrix is already compressed");
+  AS_CHECK(sub < m.items.size(), "sub-matrix id out of range");
+  const DenseItem parent = std::move(m.items[sub]);
+  const uint64_t rows = parent.max_row - parent.min_row + 1;
+  AS_CHECK(pos.size() >= 2 && pos.front() == 0 && pos.back() == rows, "division positions must span the rows of the sub-block");
+  std::vector<uint64_t> off = row_offsets(m.coo_row, parent.begin_coo, parent.end_coo + 1, parent.min_row, rows);
+  m.items.erase(m.items.begin() + (long)sub);
+  for (size_t b = 0; b + 1 < pos.size(); b++) {
+    AS_CHECK(pos[b + 1] >= pos[b], "division positions must be non-decreasing");
+    if (pos[b + 1] == pos[b] || off[pos[b]] == off[pos[b + 1]]) continue;  // "find empty row group"
+    DenseItem it;
+    it.min_row = parent.min_row + pos[b];
+    it.max_row = parent.min_row + pos[b + 1] - 1;
+    it.min_col = parent.min_col;
+    it.max_col = parent.max_col;
+    it.begin_coo = off[pos[b]];
+    it.end_coo = off[pos[b + 1]] - 1;
+    it.is_col_blocked = parent.is_col_blocked;
+    m.items.push_back(std::move(it));
+  }
+  m.is_blocked = true;
+}
+
+void fixed_len_row_div(Matrix &m, uint64_t len, uint64_t sub) {
+  AS_CHECK(len > 0, "strip height must be positive");
+  AS_CHECK(sub < m.items.size(), "sub-matrix id out of range");
+  const uint64_t rows = m.items[sub].max_row - m.items[sub].min_row + 1;
+  std::vector<uint64_t> pos;
+  for (uint64_t r = 0; r < rows; r += len) pos.push_back(r);
+  pos.push_back(rows);
+  var_len_row_div(m, pos, sub);
+}
+
+// The elements of the sub-block are regrouped band by band of `len` columns, counted from the sub-block's first
+// column, inside its own stretch of the element arrays (inside a band in their previous order); every band that
+// holds elements becomes a sub-block over the parent's rows, marked is_col_blocked.  (Upstream copies the
+// regrouped VALUES to the front of the value array instead of to the parent's stretch, op_manager.cc:955-962; here
+// they stay with their elements, which is the same thing when the parent is the first sub-block.)
+void fixed_len_col_div(Matrix &m, uint64_t len, uint64_t sub) {
+  AS_CHECK(len > 0, "band width must be positive");
+  AS_CHECK(!m.is_compressed, "matrix is already compressed");
+  AS_CHECK(sub < m.items.size(), "sub-matrix id out of range");
+  const DenseItem parent = std::move(m.items[sub]);
+  const uint64_t b0 = parent.begin_coo, n = parent.end_coo - parent.begin_coo + 1;
+  const uint64_t bands = (parent.max_col - parent.min_col + len) / len;
+  std::vector<uint64_t> begin(bands + 1, 0);
+  for (uint64_t k = b0; k < b0 + n; k++) {
+    AS_CHECK(m.coo_col[k] >= parent.min_col && m.coo_col[k] <= parent.max_col, "column outside the sub-block");
+    begin[(m.coo_col[k] - parent.min_col) / len + 1]++;
+  }
+  for (uint64_t b = 0; b < bands; b++) begin[b + 1] += begin[b];
+  std::vector<uint64_t> nrow(n), ncol(n), next(begin.begin(), begin.end() - 1);
+  ValVec nval(n);
+  for (uint64_t k = b0; k < b0 + n; k++) {
+    const uint64_t p = next[(m.coo_col[k] - parent.min_col) / len]++;
+    nrow[p] = m.coo_row[k];
+    ncol[p] = m.coo_col[k];
+    nval[p] = m.coo_val[k];
+  }
+  std::copy(nrow.begin(), nrow.end(), m.coo_row.begin() + (long)b0);
+  std::copy(ncol.begin(), ncol.end(), m.coo_col.begin() + (long)b0);
+  std::copy(nval.begin(), nval.end(), m.coo_val.begin() + (long)b0);
+  m.items.erase(m.items.begin() + (long)sub);
+  for (uint64_t b = 0; b < bands; b++) {
+    if (begin[b + 1] == begin[b]) continue;  // "find empty col group": dropped
+    DenseItem it;
+    it.is_col_blocked = true;
+    it.min_col = parent.min_col + b * len;
+    it.max_col = std::min(parent.max_col, parent.min_col + b * len + len - 1);
+    it.min_row = parent.min_row;
+    it.max_row = parent.max_row;
+    it.begin_coo = b0 + begin[b];
+    it.end_coo = b0 + begin[b + 1] - 1;
+    m.items.push_back(std::move(it));
+  }
+  m.is_blocked = true;
+}
+
 // --------------------------------------------------------------------------
 // compress_dense_view (op_manager.cc:968-1101): every dense block gets
 // --------------------------------------------------------------------------

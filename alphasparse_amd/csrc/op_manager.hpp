@@ -55,6 +55,13 @@ void fixed_len_row_div(Matrix &m, uint64_t len);
 // fixed_len_col_div (op_manager.cc:665), whole-matrix form: column bands of `len` columns, every band a
 // sub-block over all rows (is_col_blocked), bands without elements dropped
 void fixed_len_col_div(Matrix &m, uint64_t len);
+// The three divisions applied to sub-block `sub` of an already divided matrix (op_manager.cc:243-365, 808-965;
+// upstream's var_len_row_div stops with "further div is not support", :520): positions are relative to the
+// sub-block's first row, bands are counted from its first column; the parent leaves the table, its parts are
+// appended at the end.
+void var_len_row_div(Matrix &m, const std::vector<uint64_t> &block_first_row_csr_index, uint64_t sub);
+void fixed_len_row_div(Matrix &m, uint64_t len, uint64_t sub);
+void fixed_len_col_div(Matrix &m, uint64_t len, uint64_t sub);
 // compress_dense_view (op_manager.cc:968)
 void compress_dense_view(Matrix &m);
 

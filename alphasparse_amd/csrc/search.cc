@@ -7,6 +7,7 @@
 #include <fstream>
 #include <map>
 
+#include "device_facts.hpp"
 #include "hip_layer.h"
 
 namespace asx {
@@ -51,6 +52,19 @@ MatrixInfo get_sub_matrix_info_from_compressed_matrix_block(const Matrix &m, uin
           for (uint64_t e = 0; same && e < len; e++) same = col[a + e] == col[b + e];
         }
       if (same) { i.row_block = h; break; }
+    }
+    // distinct diagonals, where a row is short enough for the ELL template to be in question at all
+    if (i.max_row_nnz <= 64) {
+      const std::vector<uint64_t> &row = m.items[sub].cb->read_index[0]->index_arr.v;
+      std::vector<int64_t> seen;
+      int64_t last = INT64_MIN;
+      for (size_t k = 0; k < col.size() && seen.size() <= 64; k++) {
+        const int64_t d = (int64_t)col[k] - (int64_t)row[k];
+        if (d == last) continue;
+        last = d;
+        if (std::find(seen.begin(), seen.end(), d) == seen.end()) seen.push_back(d);
+      }
+      i.diagonals = seen.size();
     }
   }
   return i;
@@ -172,6 +186,15 @@ std::string convert_graph_to_string(const BestGraph &g) {
   return s;
 }
 
+// What upstream's main prints once the search is over (main.cc:646-657): the two figures, the graph followed by an
+// empty line (the string already ends its last line, `<< endl` adds another), or "error" when nothing ran, then
+// "finish search".
+std::string convert_search_result_to_string(float gflops, float time_ms, const BestGraph &g) {
+  char head[256];
+  snprintf(head, sizeof head, "gflops:%g\ntime:%g\n", gflops, time_ms);
+  return std::string(head) + (gflops != 0 ? convert_graph_to_string(g) + "\n" : std::string("error\n")) + "finish search\n";
+}
+
 // ---------------------------------------------------------------------------------------------
 namespace {
 
@@ -187,6 +210,7 @@ struct Ctx {
   // per row of the input: y for that x (a host CSR product computed once per search), and the same sum over the
   // magnitudes
   std::vector<double> row_sum, row_mag;
+  std::vector<uint64_t> row_len;   // elements of every row of the input
   // time per SpMV (ms) of the best whole graph measured so far, 0 before the first: a strip kernel that alone takes
   // longer cannot be part of a better graph, whichever way the strips are launched
   float best_whole_ms = 0;
@@ -212,11 +236,9 @@ void set_launch(Template &t, const TemplateNode &n) {
   if (n.tblock_num > 0) t.tblock_num = (uint64_t)n.tblock_num;
 }
 
-// time the kernels of a builder: warm-up, a short probe, then ~timed_region_ms
 // One SpMV with the search's probe vector (x[j] = 1 + j % 7): the rows that the loaded kernels cover (sub-matrix
-// `sub`, or all with sub < 0) must hold the host's product for that x, every other row of y zero.  The bound is loose (1e-3 / 1e-9 of the sum of
-// the magnitudes): it is there to catch an element that was lost, doubled or added to the wrong row, not
-// rounding.  Throws on a mismatch.
+// `sub`, or all with sub < 0) must hold the host's product for that x, every other row of y zero.  Throws on a
+// mismatch.
 void verify_candidate(Ctx &c, Builder &b, const Matrix &m, int64_t sub) {
   if (!c.opt.verify_candidates) return;
   launch_spmv(b, b.x.ptr, b.y.ptr);
@@ -230,10 +252,14 @@ void verify_candidate(Ctx &c, Builder &b, const Matrix &m, int64_t sub) {
     const DenseItem &it = m.items[(size_t)sub];
     for (uint64_t r = it.min_row; r <= it.max_row; r++) covered[m.sorted_row_index.present ? m.sorted_row_index[r] : r] = 1;
   }
-  const double tol = f64 ? 1e-9 : 1e-3;
+  // 64 roundings of the value type on the sum of the magnitudes, times the row's length up to 16 (sums of long
+  // rows are added up in trees and by atomics in any order): an element of a short row that is lost, doubled or
+  // added to another row is far outside, and so is a typical element of a row of thousands
+  const double eps64 = 64.0 * (f64 ? 2.220446049250313e-16 : 1.1920928955078125e-07);
   for (uint64_t r = 0; r < b.rows; r++) {
     const double got = f64 ? ((const double *)y.data())[r] : (double)((const float *)y.data())[r];
     const double want = covered[r] ? c.row_sum[r] : 0.0;
+    const double tol = eps64 * (double)std::min<uint64_t>(16, std::max<uint64_t>(1, c.row_len[r]));
     if (!(std::fabs(got - want) <= tol * c.row_mag[r] + 1e-30))
       throw Error("wrong result: y[" + std::to_string(r) + "] = " + std::to_string(got) + " for a row sum of " +
                   std::to_string(want));
@@ -314,7 +340,7 @@ std::vector<TemplateNode> launch_candidates(const Template &t) {
       for (long th : {1024, 512}) push(th, 1, 1);
       break;
     case SHARED_MEMORY_PRODUCT_BIN_TEMPLATE:
-      for (long th : {1024, 512, 256}) push(th, 1, 1);
+      for (long th : {1024, 512}) push(th, 1, 1);
       break;
     default:
       push(256, 1, 1);
@@ -325,7 +351,7 @@ std::vector<TemplateNode> launch_candidates(const Template &t) {
 // find_best_template_node_of_specific_sub_matrix_from_template_set (default_auto_tuner.cc:44):
 // best (template, launch parameters) for an already built format of one sub-matrix
 bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<TemplateType> &types, SearchStrategy *local,
-                        TemplateNode &best, float &best_gflops, float &best_ms) {
+                        TemplateNode &best, float &best_gflops, float &best_ms, const MatrixInfo *info = nullptr) {
   best_gflops = 0;
   best_ms = 0;
   execute_default_div_to_complete_each_level_blocking(m, sub);
@@ -338,10 +364,26 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
   for (TemplateType type : types) {
     if (!is_supported_by_template(type, m, sub)) continue;
     std::unique_ptr<Builder> b;
+    // A stencil (as many diagonals as the longest row has elements) through the ELL template: the form without a
+    // column array first, and the launch settings swept in that form -- it is what wins there, and the sooner it is
+    // measured the sooner a caller has its graph.
+    long first_form = 0;
+    // A banded matrix whose rows come in blocks with the same columns through the tile template: the form that has
+    // won on such matrices (column runs where they shorten the stream, row ownership, blocks of rows as pieces) is
+    // built and measured first; the plain form and the steps towards it follow only where it does not apply.
+    bool tile_blocks_first = false;
     try {
       b = init_code_builder(m);
-      add_template_to_builder(*b, sub, type);
-      compress_template_in_builder(*b, sub);
+      if (type == SHARED_MEMORY_TILE_TEMPLATE && info && info->row_block > 1 && is_supported_by_template(type, m, sub) &&
+          add_tile_template_variant_to_builder(*b, sub, true, true, info->row_block)) {
+        tile_blocks_first = true;
+      } else {
+        add_template_to_builder(*b, sub, type);
+        compress_template_in_builder(*b, sub);
+        if (type == DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS && info && info->diagonals > 0 &&
+            info->diagonals <= std::max<uint64_t>(1, info->max_row_nnz) && set_diagonal_columns(*b, sub))
+          first_form = 2;
+      }
       load_and_upload(*b, c.opt.device);
       if (as_hip_h2d(b->x.ptr, c.probe_x.data(), b->x.bytes) != 0) throw Error(as_hip_last_error());
     } catch (const std::exception &e) {
@@ -349,8 +391,51 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
       c.log(std::string("  candidate failed: ") + e.what());
       continue;
     }
+    if (tile_blocks_first) {
+      bool measured = false;
+      for (long threads : {1024l, 512l}) {
+        TemplateNode n;
+        n.type = type; n.thread_num_in_block = threads; n.thread_num_of_row_reduce = 1; n.vec_width = 1;
+        n.col_relative = b->subs[sub].tpl->col_runs ? 3 : 0;
+        n.own_rows = 1;
+        n.row_block = (long)info->row_block;
+        float ms = 0, gf = 0;
+        try {
+          set_launch(*b->subs[sub].tpl, n);
+          invalidate_module(*b);
+          verify_candidate(c, *b, m, (int64_t)sub);
+          time_builder(c, *b, ms, gf);
+        } catch (const std::exception &e) {
+          c.res.failed_candidates++;
+          c.log(std::string("  candidate failed: ") + e.what());
+          continue;
+        }
+        c.res.candidates++;
+        measured = true;
+        n.tblock_num = (long)b->subs[sub].tpl->tblock_num;
+        c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
+              " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
+              (n.col_relative == 3 ? " column runs," : "") + " row ownership, row blocks of " + std::to_string(n.row_block) +
+              " -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us" + c.stamp());
+        if (gf > best_gflops * (best_gflops > 0 && best.type == type ? 1.01f : 1.0f)) { best_gflops = gf; best_ms = ms; best = n; }
+        bool go = local ? continue_search(*local, gf) : true;
+        if (!go || !continue_search(c.global)) return best_gflops > 0;
+      }
+      if (measured) continue;   // the other forms of the tile template are steps towards this one
+      // it did not run: the plain form and its refinements below
+      try {
+        add_template_to_builder(*b, sub, type);
+        compress_template_in_builder(*b, sub);
+        load_and_upload(*b, c.opt.device);
+      } catch (const std::exception &e) {
+        c.res.failed_candidates++;
+        c.log(std::string("  candidate failed: ") + e.what());
+        continue;
+      }
+    }
     for (TemplateNode n : launch_candidates(*b->subs[sub].tpl)) {
       float ms = 0, gf = 0;
+      n.col_relative = first_form;
       try {
         set_launch(*b->subs[sub].tpl, n);
         invalidate_module(*b);
@@ -367,7 +452,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
       c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
             " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) + " row_reduce " +
             std::to_string(n.thread_num_of_row_reduce) + " vec " + std::to_string(n.vec_width) + " -> " + std::to_string(gf) +
-            " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
+            (first_form == 2 ? " diagonal columns" : "") + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
       // another launch setting of the template that leads must lead by more than the noise of two timings (1 %):
       // the same matrix then gets the same graph from one search to the next
       const bool same_template = best_gflops > 0 && best.type == type;
@@ -380,7 +465,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
     }
     // the best launch of the ELL template once more with 16-bit relative columns and then with the columns
     // computed from the slots' diagonals, where the matrix allows them
-    if (type == DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS && best.type == type && best_gflops > 0) {
+    if (type == DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS && first_form == 0 && best.type == type && best_gflops > 0) {
       const TemplateNode launch = best;
       for (long form : {1l, 2l}) {
         try {
@@ -644,7 +729,7 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
     Skeleton s;
     s.name = "S10";
     s.templates = {SHARED_MEMORY_X_SLICE_TEMPLATE};
-    long slice = (long)(131072 / (info.is_double ? 8 : 4));
+    long slice = (long)(x_slice_bytes() / (info.is_double ? 8 : 4));
     s.knobs = [](ParamEnumerator &e, long *k) { e.add(&k[0], 0, 0, 1); };
     s.nodes = [slice](const long *) {
       return std::vector<StrategyNode>{make_strategy(COMPRESSED_TBLOCK_LEVEL_COL_DIV_COL_SLICE_PARAM_STRATEGY, slice)};
@@ -659,7 +744,7 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
     Skeleton s;
     s.name = "S11";
     s.templates = {SHARED_MEMORY_TILE_TEMPLATE};
-    long slice = (long)(131072 / (info.is_double ? 8 : 4)), group = slice / 4;
+    long slice = (long)(x_slice_bytes() / (info.is_double ? 8 : 4)), group = slice / 4;
     // rows that come in blocks of equal columns: row groups of whole blocks (halved groups too), so that the
     // template can store a block of rows as one piece
     if (info.row_block > 1) group = group / (2 * (long)info.row_block) * (2 * (long)info.row_block);
@@ -670,33 +755,36 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
     };
     return s;
   };
-  // the same tiles in two passes (products streamed to scratch, then summed in small groups of rows): for
-  // rows too short to leave several elements per slice, where every x read of a row-wise kernel would
-  // bring a cache line from HBM.  k0: slice width = 128 KB of x, a quarter or a 32nd of it (narrow slices:
-  // several first-pass workgroups per CU, but shorter runs of products); k1: row group height 65536 or
-  // 8192 (the area the products of one slice trip are written to; the tall one first, it has won on every
-  // matrix measured so far and a search that runs out of time should have seen it).
+  // the same elements in two passes (products streamed to scratch band by band of y, then summed band by band):
+  // for rows too short to leave several elements per slice, where every x read of a row-wise kernel would
+  // bring a cache line from HBM.  k0: slice width = 64, 128 or 32 KB of x (narrow slices: several first-pass
+  // workgroups per CU, but shorter runs of products; C3: first pass 12.4 / 14.6 / 13.2 us, C5: 69.8 with 64 KB
+  // against 66.0 with 128); k1: bands of 4096 or 2048 rows of y (C3: second pass 10.8 / 10.9 us, first pass
+  // 13.2 / 14.7; 8192 rows: second pass 12.2).
   auto S12 = [&]() {
     Skeleton s;
     s.name = "S12";
     s.templates = {SHARED_MEMORY_PRODUCT_BIN_TEMPLATE};
-    long slice = (long)(131072 / (info.is_double ? 8 : 4));
+    long slice = (long)(x_slice_bytes() / (info.is_double ? 8 : 4));
     s.knobs = [](ParamEnumerator &e, long *k) {
       e.add(&k[0], 0, 2, 1);
       e.add(&k[1], 0, 1, 1);
     };
     s.nodes = [slice](const long *k) {
-      static const int shift[] = {0, 2, 5};
+      static const int shift[] = {1, 0, 2};
       return std::vector<StrategyNode>{make_strategy(COMPRESSED_TBLOCK_LEVEL_COL_DIV_ROW_GROUP_COL_SLICE_PARAM_STRATEGY,
-                                                     slice >> shift[k[0]], k[1] ? 8192 : 65536, 8192)};
+                                                     slice >> shift[k[0]], k[1] ? 2048 : 4096, 8192)};
     };
     return s;
   };
+  // a stencil (no more diagonals than the longest row has elements): ELL first, its diagonal form is what wins
+  const bool stencil = info.diagonals > 0 && info.diagonals <= (uint64_t)std::max(1l, mx);
+  if (stencil && mx <= 512) out.push_back(S5());
   {
-    long vs = info.is_double ? 8 : 4, slice = 131072 / vs;
+    long vs = info.is_double ? 8 : 4, slice = x_slice_bytes() / vs;
     long slices = ((long)info.col_num + slice - 1) / slice;
-    if (slices >= 2 && (long)info.col_num * vs > (4l << 20) && mx <= 64) out.push_back(S12());
-    if (slices >= 2 && (long)info.col_num * vs > (4l << 20) && avg >= std::max(8l, slices / 4)) out.push_back(S11());
+    if (slices >= 2 && (long)info.col_num * vs > (long)kL2BytesPerXcd && mx <= 64) out.push_back(S12());
+    if (slices >= 2 && (long)info.col_num * vs > (long)kL2BytesPerXcd && avg >= std::max(8l, slices / 4)) out.push_back(S11());
     if (mn >= 32 * slices && slices >= 2) out.push_back(S10());
   }
   // The two general templates (outside upstream's white list; SearchOptions::general_templates): every
@@ -738,7 +826,7 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
   if (general_templates && mx <= 512) { out.push_back(G1()); out.push_back(G2()); }
   // order tried upstream: 8, 1, 5, 9, 4, 6, 7, 2, 3
   if (mn >= 128) out.push_back(S8());
-  if (mx <= 512) { out.push_back(S1()); out.push_back(S5()); }
+  if (mx <= 512) { out.push_back(S1()); if (!stencil) out.push_back(S5()); }
   if (!globally_sorted) out.push_back(S9());
   if (mn >= 30 && mx <= 512) out.push_back(S4());
   if (mn >= 32 && mx <= 1024) { out.push_back(S6()); out.push_back(S7()); }
@@ -786,7 +874,7 @@ bool find_best_path_of_compressed_sub_matrix(Ctx &c, const Matrix &base, uint64_
       float gf = 0, ms = 0;
       bool ok = false;
       try {
-        ok = find_best_template(c, *m, sub, sk.templates, &local, tn, gf, ms);
+        ok = find_best_template(c, *m, sub, sk.templates, &local, tn, gf, ms, &info);
       } catch (const std::exception &ex) {
         c.res.failed_candidates++;
         c.log(std::string("  candidate failed: ") + ex.what());
@@ -910,6 +998,14 @@ BuiltGraph build_from_graph(const CooInput &in, const BestGraph &g, unsigned wav
   r.builder = init_code_builder(*r.matrix);
   r.builder->serial_launch = g.serial_launch;
   for (size_t s = 0; s < g.subs.size(); s++) {
+    if (g.subs[s].tpl.type == SHARED_MEMORY_TILE_TEMPLATE && g.subs[s].tpl.own_rows == 1 && g.subs[s].tpl.row_block > 1) {
+      // built at once, the way the search built it
+      AS_CHECK(add_tile_template_variant_to_builder(*r.builder, s, g.subs[s].tpl.col_relative == 3, true, (uint64_t)g.subs[s].tpl.row_block) &&
+                   r.builder->subs[s].tpl->col_runs == (g.subs[s].tpl.col_relative == 3),
+               "the best graph's tile template cannot be rebuilt");
+      set_launch(*r.builder->subs[s].tpl, g.subs[s].tpl);
+      continue;
+    }
     add_template_to_builder(*r.builder, s, g.subs[s].tpl.type);
     compress_template_in_builder(*r.builder, s);
     if (g.subs[s].tpl.col_relative == 1)
@@ -933,6 +1029,9 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
   AS_CHECK(!empty_rows || opt.remove_empty_rows, "input must not have rows without elements");
   SearchResult res;
   Ctx c{opt, res, init_search_strategy(opt.struggle_step_num, opt.total_time_s), {}};
+  // the formats are sized for the GPU the candidates run on
+  if (as_hip_init(opt.device) != 0) throw Error(as_hip_last_error());
+  read_device_facts(opt.device);
   c.empty_rows = empty_rows;
   if (empty_rows) c.log("rows without elements are removed before the first operator of every graph");
   size_t cols = in.col_index_max + 1;
@@ -946,8 +1045,10 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
   if (opt.verify_candidates) {
     c.row_sum.assign(in.row_index_max + 1, 0.0);
     c.row_mag.assign(in.row_index_max + 1, 0.0);
+    c.row_len.assign(in.row_index_max + 1, 0);
     for (size_t i = 0; i < in.row.size(); i++) {
       const double xj = 1.0 + (double)(in.col[i] % 7);
+      c.row_len[in.row[i]]++;
       c.row_sum[in.row[i]] += in.val[i] * xj;
       c.row_mag[in.row[i]] += std::fabs(in.val[i]) * xj;
     }
@@ -1006,7 +1107,7 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
   // winner is then known early (it is what a caller waits for), and it bounds what strategies 1 and 2 still sweep.
   // It leaves them a fifth of the budget.
   const bool sort_first = opt.only_dense_strategy == 0 && !one_strip_only &&
-                          in.col_index_max + 1 > (4ull << 20) / (in.val_dtype == DOUBLE ? 8 : 4) &&
+                          in.col_index_max + 1 > kL2BytesPerXcd / (in.val_dtype == DOUBLE ? 8 : 4) &&
                           longest_row >= 64 * std::max<uint64_t>(1, in.row.size() / row_len.size());
   // strategy 1: INPUT -> COMPRESS (a tenth of the budget, :5092)
   auto strategy1 = [&]() {
@@ -1041,8 +1142,8 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
       // `lowest` elements and the rest -- which is what the LDS-tile kernel wants when x is larger
       // than an XCD's L2 cache; then the upstream grid 512/128/32 x 4/8/16 with bands up to 2048.
       std::vector<std::array<long, 3>> bands;
-      if (in.col_index_max + 1 > (4ull << 20) / (in.val_dtype == DOUBLE ? 8 : 4))
-        for (long low : {16, 64, 256}) bands.push_back({low, low, 2});
+      if (in.col_index_max + 1 > kL2BytesPerXcd / (in.val_dtype == DOUBLE ? 8 : 4))
+        for (long low : {64, 16, 256}) bands.push_back({low, low, 2});
       for (long low : {512, 128, 32})
         for (long rate : {4, 8, 16}) bands.push_back({low, 2048, rate});
       std::vector<std::vector<uint64_t>> seen;
@@ -1106,9 +1207,7 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
   }
   res.seconds = now_s();
   AS_CHECK(res.best.gflops > 0, "the search found no working candidate");
-  char head[256];
-  snprintf(head, sizeof head, "gflops:%g\ntime:%g\n", res.best.gflops, res.best.time_ms);
-  res.log += std::string(head) + convert_graph_to_string(res.best) + "finish search\n";
+  res.log += convert_search_result_to_string(res.best.gflops, res.best.time_ms, res.best);
   return res;
 }
 

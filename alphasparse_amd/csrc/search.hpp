@@ -21,6 +21,10 @@ struct MatrixInfo {
   // 4, 3 or 2 where the first rows come in blocks of that many consecutive rows with the same columns (the dense
   // blocks of a FEM matrix), else 1; only get_sub_matrix_info_from_compressed_matrix_block fills it
   uint64_t row_block = 1;
+  // distinct diagonals (column - row) the elements lie on, counted up to 65 (65 = more); 0 = not counted (rows of
+  // more than 64 elements); only get_sub_matrix_info_from_compressed_matrix_block fills it.  A stencil has as many
+  // as its longest row has elements: the ELL template then needs no column array at all.
+  uint64_t diagonals = 0;
 };
 MatrixInfo get_matrix_info(const Matrix &m);                                      // matrix_info.cc:22
 MatrixInfo get_sub_matrix_info_from_compressed_matrix_block(const Matrix &m, uint64_t sub);  // matrix_info.cc:140
@@ -86,6 +90,8 @@ struct BestGraph {
 // convert_dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_to_string_safety
 // (whilte_list_path_impl.cc:4150)
 std::string convert_graph_to_string(const BestGraph &g);
+// the lines upstream's main prints around it (main.cc:646-657), up to and including "finish search"
+std::string convert_search_result_to_string(float gflops, float time_ms, const BestGraph &g);
 
 struct SearchOptions {
   double total_time_s = 120;        // upstream: 32400

@@ -203,6 +203,7 @@ AS_DECLARE_TEMPLATE(tpl_shared_memory_total_warp_reduce)
 AS_DECLARE_TEMPLATE(tpl_direct_atom_total_warp_reduce)
 AS_DECLARE_TEMPLATE(tpl_unaligned_warp_reduce)
 AS_DECLARE_TEMPLATE(tpl_unaligned_warp_reduce_with_warp_reduce)
+AS_DECLARE_TEMPLATE(tpl_empty)
 AS_DECLARE_TEMPLATE(tpl_shared_memory_x_slice)
 AS_DECLARE_TEMPLATE(tpl_shared_memory_tile)
 AS_DECLARE_TEMPLATE(tpl_shared_memory_product_bin)

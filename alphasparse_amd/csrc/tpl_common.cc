@@ -96,6 +96,7 @@ void init_template_common(Template &t, TemplateType type, const Matrix &m, uint6
 
 bool template_needs_cleared_y(const Template &t, const Matrix &m, uint64_t sub) {
   if (t.is_atom_add) return true;
+  if (t.type == EMPTY_TEMPLATE) return true;  // no kernel: the clear is what writes the rows of this sub-matrix
   // the CSR5-like pair adds the partial sums of rows that cross a tile or a wavefront into y
   if (t.type == UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE ||
       t.type == UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE_WITH_WARP_REDUCE)
@@ -103,8 +104,9 @@ bool template_needs_cleared_y(const Template &t, const Matrix &m, uint64_t sub) 
   // the two-kernel LDS templates store every row of the strip in their finish kernel, with or without elements
   if (t.finish_tblock_num && (t.type == SHARED_MEMORY_TILE_TEMPLATE || t.type == SHARED_MEMORY_PRODUCT_BIN_TEMPLATE))
     return false;
-  // the tile template under row ownership stores every row of every row group, zeros included
-  if (t.type == SHARED_MEMORY_TILE_TEMPLATE && t.own_rows) return false;
+  // the tile template under row ownership stores every row of every row group that holds an element, zeros
+  // included; a row group without any element has no run and is stored by nobody
+  if (t.type == SHARED_MEMORY_TILE_TEMPLATE && t.own_rows) return t.sc("row_groups_without_elements") != 0;
   // the row-wise templates store the rows that have a unit (TLB, WLB or BLB): a row without elements has none
   const DenseItem &it = m.items[sub];
   const uint64_t sub_rows = it.max_row - it.min_row + 1;
@@ -131,6 +133,7 @@ bool template_needs_cleared_y(const Template &t, const Matrix &m, uint64_t sub) 
     case UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE: return tpl_unaligned_warp_reduce::call;          \
     case UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE_WITH_WARP_REDUCE:                                 \
       return tpl_unaligned_warp_reduce_with_warp_reduce::call;                                          \
+    case EMPTY_TEMPLATE: return tpl_empty::call;                                                        \
     case SHARED_MEMORY_X_SLICE_TEMPLATE: return tpl_shared_memory_x_slice::call;                        \
     case SHARED_MEMORY_TILE_TEMPLATE: return tpl_shared_memory_tile::call;                              \
     case SHARED_MEMORY_PRODUCT_BIN_TEMPLATE: return tpl_shared_memory_product_bin::call;                \

@@ -39,6 +39,7 @@
 // Row blocks (init_variant(..., row_block = b), under row ownership): where b consecutive rows hold the same
 // columns (the dense b x b blocks of a FEM matrix), a block of rows is one piece: columns, lane word and reads of
 // x are those of its first row, an element is b values, and a lane adds into b sums.
+#include "device_facts.hpp"
 #include "templates.hpp"
 
 namespace asx {
@@ -46,8 +47,6 @@ namespace tpl_shared_memory_tile {
 
 static const unsigned kLaneRuns = 4;        // column runs a lane of the column-run form can hold
 
-static const uint64_t kLdsBytes = 163840;   // LDS of one CU
-static const uint64_t kCuNum = 256;
 static const uint64_t kLaneElems = 8;       // consecutive elements of one lane in a wavefront step
 static const uint64_t kRunUnit = 64 * kLaneElems;  // elements of one wavefront step
 static const unsigned kNewPieceBit = 14;    // lane word: bit 14 + j = element j (1..7) starts a new piece
@@ -60,7 +59,7 @@ bool is_supported(const Matrix &m, uint64_t sub) {
   const DenseItem &it = m.items[sub];
   const CompressedBlock &cb = *it.cb;
   const uint64_t S = cb.col_slice, R = cb.row_group, vs = (uint64_t)dtype_size(m.val_dtype);
-  if (S == 0 || R == 0 || S > 65536 || R > 32768 || S % 4 || (S + R) * vs > kLdsBytes) return false;
+  if (S == 0 || R == 0 || S > 65536 || R > 32768 || S % 4 || (S + R) * vs > device_facts().lds_bytes) return false;
   if (it.max_row != cb.read_index[0]->max_row) return false;  // not after COMPRESSED_ROW_PADDING
   const Index &bl = *cb.read_index[2];
   const std::vector<uint64_t> &row = cb.read_index[0]->index_arr.v, &col = cb.read_index[1]->index_arr.v;
@@ -186,7 +185,7 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
     blk_cost[b] = (bl.coo_begin[b + 1] - bl.coo_begin[b]) * elem_bytes + pieces * piece_cost;
   }
   // one trip per workgroup the 256 CUs hold at a time with this much LDS each
-  uint64_t want = kCuNum * std::max<uint64_t>(1, kLdsBytes / ((S + R) * vs));
+  uint64_t want = device_facts().cu_num * std::max<uint64_t>(1, device_facts().lds_bytes / ((S + R) * vs));
   want = std::max<uint64_t>(1, std::min<uint64_t>(want, (n + 16383) / 16384));
   std::vector<uint64_t> group_first_block{0};
   // Row ownership (own_rows): the elements are taken row group by row group and a trip is a whole number of row
@@ -264,8 +263,15 @@ static std::unique_ptr<Template> build(const Matrix &m, uint64_t sub, bool colum
       }
     }
     group_first_own_run[NG] = runs.size();
+    // A row group without elements has no run: the workgroup that owns it never reaches the group's stores, and
+    // its rows of y are then written by nobody (template_needs_cleared_y asks for the clear of y)
+    uint64_t groups_without_run = 0;
     for (uint64_t g = NG; g-- > 0;)
-      if (group_cost[g] == 0) group_first_own_run[g] = group_first_own_run[g + 1];  // a row group without elements
+      if (group_cost[g] == 0) {
+        group_first_own_run[g] = group_first_own_run[g + 1];
+        groups_without_run++;
+      }
+    t->scalar["row_groups_without_elements"] = groups_without_run;
     if (runs.size() * slice_cost * 4 > stream_cost) return nullptr;
     uint64_t total = 0;
     for (uint64_t c : group_cost) total += c;

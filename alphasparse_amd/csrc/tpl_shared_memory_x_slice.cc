@@ -10,6 +10,7 @@
 // consecutive elements per unit, 128-bit value loads), sums each unit over its 16 lanes with DPP row
 // operations and adds it to the unit's row with one atomic (rows are shared between slices and
 // units, so y is always accumulated atomically).  No per-BLB control flow, no dependent loads.
+#include "device_facts.hpp"
 #include "templates.hpp"
 
 namespace asx {
@@ -17,7 +18,7 @@ namespace tpl_shared_memory_x_slice {
 
 // largest slice whose values fit the LDS budget of one workgroup (128 KB; 32 KB stay free)
 static const unsigned kBatch = 4;  // steps of 4 units whose loads a wavefront keeps in flight together
-static uint64_t max_slice(DType val_dtype) { return 131072 / (uint64_t)dtype_size(val_dtype); }
+static uint64_t max_slice(DType val_dtype) { return x_slice_bytes() / (uint64_t)dtype_size(val_dtype); }
 
 bool is_supported(const Matrix &m, uint64_t sub) {
   const DenseItem &it = m.items[sub];

@@ -25,6 +25,8 @@ def _bind_search(L):
     L.as_search_log.restype = C.c_char_p
     L.as_search_log.argtypes = [vp]
     L.as_search_stats.argtypes = [vp, C.POINTER(C.c_double)]
+    L.as_search_best_graph.restype = C.c_int64
+    L.as_search_best_graph.argtypes = [vp, capi.longp, C.c_uint64]
     L.as_search_build_best.restype = vp
     L.as_search_build_best.argtypes = [vp, vp]
     L.as_part_execute_code_builder.argtypes = [vp, C.POINTER(C.c_int64), C.c_uint64, C.c_uint64, C.POINTER(C.c_float),
@@ -44,6 +46,13 @@ class SearchResult:
          self.n_sub, self.dense_strategy) = [float(x) for x in out]
         self.report = self._L.as_search_report(handle).decode()
         self.log = self._L.as_search_log(handle).decode()
+
+    def best_graph(self):
+        """The best graph as the flat list of numbers that as_graph_report takes."""
+        n = capi.check(self._L.as_search_best_graph(self._h, None, 0))
+        d = (C.c_long * n)()
+        capi.check(self._L.as_search_best_graph(self._h, d, n))
+        return list(d)
 
     def build_best(self):
         """Rebuild the best format from the input matrix -> Builder (not yet uploaded)."""

@@ -15,9 +15,12 @@ C5 extreme irregularity), each with its GFLOP/s, roofline fraction (also on the 
 tuning time, result check and CPU baseline.  C2, C5 and C1 are always searched; C3 and C4 are searched while the
 wall-clock budget (--budget-seconds) allows and otherwise run the committed winners of earlier searches
 (`tuning.mode` says which); a configuration that no longer fits the budget is recorded as skipped.
-With --workload only that configuration is measured and it is the headline.  With more than one row strip the
-roofline object is quoted on the strip kernel that takes the longest, timed alone, and "kernels" lists every
-strip kernel.
+With --workload only that configuration is measured and it is the headline.  The roofline object is quoted on the
+whole SpMV; with more than one row strip `roofline.dominant_kernel` holds the strip kernel that takes the longest,
+timed alone, and "kernels" lists every strip kernel.  Two byte counts are given side by side: `algorithmic_bytes` /
+`frac` count what the chosen format moves, the intermediate arrays its kernels write and read back included
+(products, row sums: `scratch_bytes`, counted twice); `algorithmic_bytes_arrays_x_y` / `frac_arrays_x_y` count the
+format arrays, x once and y once only (twice where y is cleared first).
 
 Prints ONE JSON line (rank 0).  One GPU only: --gpus above 1 exits with a message."""
 import argparse
@@ -52,18 +55,20 @@ WORKLOADS = {
 # the rocprofv3 summary that covers each configuration's kernels
 PROFILE_OF = {"C2": "profiles/spmv_ell_c2_laplacian_hbm_traffic.txt", "C3": "profiles/spmv_tile_product_bin_c3_power_law.txt",
               "C4": "profiles/spmv_tile_c4_fem_blocks.txt", "C5": "profiles/spmv_tile_product_bin_c5_extreme_irregular.txt"}
-# HBM bytes per launch of the kernel the roofline object is quoted on, measured with rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (two runs, each scaled by what the same counter reads for the plain copy kernel of
-# --copy-calibration).  Keyed by the first 16 hex digits of the SHA-256 of the generated module source: a graph
-# whose kernels changed in any way since it was profiled reports null and names the profile instead.
-MEASURED_TRAFFIC = {
-    "ff84531ca565a608": 117580800,    # C2, ELL kernel in diagonal form (pin S5,256,1,dia)
-    "e9afcd580f447551": 197734396,    # C3, tile kernel of the long strip + its finish (pin sort+div64|T1@1024|T2:slice=8192,group=65536@512)
-    "dad308d7a3b7a127": 711696691,    # C4, tile kernel, column runs, row ownership, blocks of 3 rows (pin |T1:slice=16384,group=4092@1024,runs,own,blk3)
-    "3b570d6d4c746c50": 803162829,    # C4, the same without row blocks (pin |T1:slice=16384,group=4096@1024,runs,own)
-    "4f3d4599ea632134": 701548339,    # C5, the same graph with the thread counts the search picks (tile @512, product-bin @1024)
-    "b9791554820cbb6f": 688027956,    # C5, product-bin kernel, both passes (pin sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256)
-}
+# HBM bytes per launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same
+# counter reads for the plain copy kernel of --copy-calibration), by the first 16 hex digits of the SHA-256 of the
+# generated module source: a graph whose kernels changed in any way since it was profiled reports null and names the
+# profile instead.  The figures live beside the summaries they come from.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic_by_graph_hash.json")
+
+
+def measured_traffic(graph_hash):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(graph_hash)
+    except (OSError, ValueError):
+        return None
+    return entry["bytes"] if entry else None
 
 
 def cpu_baseline(rows, r, c, v, x, nnz, seconds):
@@ -214,18 +219,39 @@ def measure(key, steps, warmup, tune_seconds, pin, cpu_seconds, copy_calibration
         us = ms * 1e3 / reps
         kb = fmt_bytes + cols * vs + strip_rows * vs * (2 if atom else 1)
         kernels.append({"sub_matrix": s, "kernel_us": round(us, 3), "algorithmic_bytes": kb,
-                        "achieved_gbs": round(kb / us / 1e3, 1), "strip_rows": strip_rows})
+                        "scratch_bytes": b.scratch_bytes(s), "algorithmic_bytes_arrays_x_y": kb - 2 * b.scratch_bytes(s),
+                        "achieved_gbs": round(kb / us / 1e3, 1), "frac": round(kb / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "frac_arrays_x_y": round((kb - 2 * b.scratch_bytes(s)) / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "strip_rows": strip_rows})
         try:  # templates with two kernels: each launched alone
             kernels[-1]["pass_us"] = [round(b.time_sub_matrix_pass(s, which, reps) * 1e3 / reps, 3) for which in (1, 2)]
         except A.AlphaSparseError:
             pass
     dominant = max(kernels, key=lambda k: k["kernel_us"])
-    if len(kernels) > 1:
-        achieved, roof_us, roof_bytes = dominant["achieved_gbs"], dominant["kernel_us"], dominant["algorithmic_bytes"]
-    else:
-        roof_us, roof_bytes = per_launch_s * 1e6, bytes_per_step
+    roof_us, roof_bytes = per_launch_s * 1e6, bytes_per_step
     csr_floor = nnz * (v.dtype.itemsize + 4) + (rows + 1) * 4 + (rows + cols) * v.dtype.itemsize
     sync_ok, sync_ms, sync_gf = A.part_execute_code_builder(b, [], 200)
+    # the product calls on device buffers of the caller, wall clock per call: the blocking call (a wait per SpMV)
+    # and the enqueue-only call (N calls, one wait)
+    dx, dy = A.DeviceArray(x), A.DeviceArray(np.zeros(rows, v.dtype))
+    calls = 300
+    for _ in range(20):
+        b.spmv_device_async(dx, dy, None)
+    b.sync()
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        b.spmv_device_async(dx, dy, None)
+        b.sync()
+    per_call_sync_us = (time.perf_counter() - t0) / calls * 1e6
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        b.spmv_device_async(dx, dy, None)
+    b.sync()
+    per_call_async_us = (time.perf_counter() - t0) / calls * 1e6
+    dx.free()
+    dy.free()
+    scratch = b.scratch_bytes()
+    bytes_arrays_x_y = bytes_per_step - 2 * scratch
 
     templates = [b.describe(s)["template"] for s in range(int(res.n_sub))]
     launches = [b.get_launch(s) for s in range(int(res.n_sub))]
@@ -257,14 +283,24 @@ def measure(key, steps, warmup, tune_seconds, pin, cpu_seconds, copy_calibration
                    "clears_y": b.clears_y(), "graph_hash": graph_hash},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(graph_hash), "traffic_profile": PROFILE_OF.get(key),
+                     "traffic": measured_traffic(graph_hash), "traffic_profile": PROFILE_OF.get(key),
                      "kernel_us": round(roof_us, 3), "algorithmic_bytes": roof_bytes,
-                     "kernel": "spmv_%d (%s)" % (dominant["sub_matrix"], templates[dominant["sub_matrix"]]),
+                     "scratch_bytes": scratch, "algorithmic_bytes_arrays_x_y": bytes_arrays_x_y,
+                     "frac_arrays_x_y": round(bytes_arrays_x_y / per_launch_s / 1e9 / HBM_PEAK_GBS, 4),
+                     "kernel": "whole SpMV: " + " + ".join("spmv_%d (%s)" % (s_, templates[s_]) for s_ in range(int(res.n_sub))),
+                     "dominant_kernel": {"kernel": "spmv_%d (%s)" % (dominant["sub_matrix"], templates[dominant["sub_matrix"]]),
+                                         "kernel_us": dominant["kernel_us"], "algorithmic_bytes": dominant["algorithmic_bytes"],
+                                         "achieved": dominant["achieved_gbs"], "frac": dominant["frac"],
+                                         "frac_arrays_x_y": dominant["frac_arrays_x_y"]},
                      "csr_floor_bytes": csr_floor,
                      "csr_floor_frac": round(csr_floor / per_launch_s / 1e9 / HBM_PEAK_GBS, 4)},
         "whole_spmv": {"us": round(per_launch_s * 1e6, 3), "algorithmic_bytes": bytes_per_step,
                        "achieved_gbs": round(whole_gbs, 1), "frac": round(whole_gbs / HBM_PEAK_GBS, 4),
+                       "algorithmic_bytes_arrays_x_y": bytes_arrays_x_y,
+                       "frac_arrays_x_y": round(bytes_arrays_x_y / per_launch_s / 1e9 / HBM_PEAK_GBS, 4),
                        "kernel_gflops": round(2.0 * nnz / per_launch_s / 1e9, 2)},
+        "per_call_us": {"kernels": round(per_launch_s * 1e6, 3), "blocking_call": round(per_call_sync_us, 3),
+                        "enqueue_only_call": round(per_call_async_us, 3), "calls": calls},
         "kernels": kernels,
         "tuning": {"mode": "pinned" if pin else "search", "seconds": round(tune_s, 2),
                    "seconds_to_best": round(res.seconds_to_best, 2),
@@ -291,8 +327,11 @@ def per_matrix_entry(key, full):
          "graph": {k: full["config"][k] for k in ("dense_strategy", "sub_matrices", "template", "launch", "columns",
                                                    "rows_owned", "row_block", "clears_y", "graph_hash", "pinned")},
          "roofline": {k: full["roofline"][k] for k in ("frac", "achieved", "kernel", "kernel_us", "algorithmic_bytes",
-                                                       "csr_floor_bytes", "csr_floor_frac", "traffic", "traffic_profile")},
-         "whole_spmv": full["whole_spmv"], "kernels": full["kernels"], "tuning": full["tuning"], "check": full["check"]}
+                                                       "scratch_bytes", "algorithmic_bytes_arrays_x_y", "frac_arrays_x_y",
+                                                       "dominant_kernel", "csr_floor_bytes", "csr_floor_frac", "traffic",
+                                                       "traffic_profile")},
+         "whole_spmv": full["whole_spmv"], "per_call_us": full["per_call_us"], "kernels": full["kernels"],
+         "tuning": full["tuning"], "check": full["check"]}
     if "cpu_baseline" in full:
         e["cpu_baseline"] = full["cpu_baseline"]
     return e

@@ -278,9 +278,19 @@ int as_builder_spmv(as_builder *b, const void *x_host, void *y_host);
 int as_builder_spmv_device(as_builder *b, const void *x_dev, void *y_dev);
 /* 1 when an SpMV of the builder's current templates starts with a clear of y, 0 when it does not; <0 error */
 int as_builder_clears_y(as_builder *b);
-/* No counterpart in the reference.  as_builder_spmv_device for callers that cannot allocate device memory (code
- * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the call compiles, loads and
- * allocates nothing.  The builder must have been uploaded and not changed since (else an error), and the scratch
+/* Enqueue only: the launches of as_builder_spmv_device on a stream of the caller (a hipStream_t passed as a plain
+ * pointer; NULL = HIP's default stream), no wait for the GPU -- the loop of the reference's generated program,
+ * which launches spmv_<id><<<..., stream>>> repetition after repetition and synchronises once
+ * (code_builder.cc:1517-1557).  With concurrent strip kernels (serial launch off) the strips' own streams fork from
+ * and join the caller's stream by events.  The call may compile and load the module when the builder changed since
+ * its upload (then it is no call for a capturing stream); as_builder_spmv_device is this call on the builder's own
+ * stream (as_builder_stream) followed by a wait for that stream. */
+int as_builder_spmv_device_async(as_builder *b, const void *x_dev, void *y_dev, void *stream);
+/* the builder's own stream (a hipStream_t), on which the blocking calls and the timing calls launch */
+void *as_builder_stream(as_builder *b);
+/* No counterpart in the reference.  as_builder_spmv_device for callers that cannot allocate device memory (tight
+ * serving loops, harnesses that forbid hipMalloc; code under HIP graph capture uses the _async twin below, since
+ * this one waits for the GPU): the call compiles, loads and allocates nothing.  The builder must have been uploaded and not changed since (else an error), and the scratch
  * arrays of its kernels (row sums of a sorted tile strip, the products of the product-bin template) are 256-byte
  * aligned pieces of one static device array of AS_STATIC_SCRATCH_BYTES that the library holds on every GPU it has
  * uploaded to, until the process ends.  A graph whose kernels need more scratch than that
@@ -289,6 +299,11 @@ int as_builder_clears_y(as_builder *b);
  * by a fill kernel at the start of the call): calls that overlap on one GPU race. */
 #define AS_STATIC_SCRATCH_BYTES (64u << 20)
 int as_builder_spmv_device_no_alloc(as_builder *b, const void *x_dev, void *y_dev);
+/* the same, enqueued on a stream of the caller without waiting for the GPU: nothing is compiled, loaded or
+ * allocated and y and the scratch pieces are cleared by fill kernels (no memset node), so the call can be recorded
+ * by a stream capture and replayed as a HIP graph (x_dev, y_dev and the builder's arrays must then stay where they
+ * are).  Same limits and the same shared static array as above. */
+int as_builder_spmv_device_no_alloc_async(as_builder *b, const void *x_dev, void *y_dev, void *stream);
 /* bytes of the static scratch array the kernels of the builder's current templates would use (0: none) */
 int64_t as_builder_static_scratch_need(as_builder *b);
 /* 0 (default): the kernels of the sub-matrices run concurrently, one stream each (code_builder.cc:1517-1518);
@@ -315,13 +330,27 @@ int as_builder_time_sub_matrix_pass(as_builder *b, int64_t sub, int pass, uint64
 /* The library keeps the code objects it compiled in this process, by module source (no counterpart in the
  * reference, which compiles every candidate with nvcc from a file: code_builder.cc:1463-1500): entries held and compilations answered from them. */
 int as_kernel_cache_stats(uint64_t *entries, uint64_t *hits);
+/* What the format builders and the search assume about the GPU: compute units, LDS a workgroup may take (both
+ * read from the GPU at the first upload or search, which refuse a GPU that is not a gfx950; MI355X values until
+ * then), XCDs and L2 bytes per XCD (fixed for gfx950).  The reference keeps the like in global_config.json
+ * (e.g. its thread and shared-memory limits read by default_auto_tuner.cc).  from_device: 1 once read or set. */
+int as_device_facts(uint64_t *cu_num, uint64_t *lds_bytes, uint64_t *xcd_num, uint64_t *l2_bytes_per_xcd, int *from_device);
+/* read them from GPU `device` now (done implicitly by upload and search) */
+int as_device_facts_read(int device);
+/* formats for a GPU that cannot be asked (another partition mode; tests): 0 keeps a value */
+int as_device_facts_set(uint64_t cu_num, uint64_t lds_bytes);
 /* fill the builder's own x (used by the timing calls) */
 int as_builder_set_x(as_builder *b, const void *x_host);
 /* `reps` launches timed with events; gflops = 2 * origin_nnz * reps / time (code_builder.cc:1557).
  * sync_each_launch = 1 reproduces the upstream loop "kernel; cudaDeviceSynchronize" (code_builder.cc:1524-1557). */
 int as_builder_time(as_builder *b, uint64_t reps, int sync_each_launch, float *time_ms, float *gflops);
-/* bytes one SpMV moves with the chosen format: padded col+val, passed metadata, x once, y once (twice with atomics) */
+/* bytes one SpMV moves with the chosen format: padded col+val, passed metadata, the kernels' scratch arrays written
+ * and read back (2 x as_builder_scratch_bytes), x once, y once (twice where y is cleared first) */
 int64_t as_builder_algorithmic_bytes(as_builder *b);
+/* bytes of the scratch arrays of the kernels of sub-matrix `sub` (-1: of all): intermediate results the kernels write
+ * and read back (products, row sums), which the format's own bytes count twice and a count of the format arrays,
+ * x and y alone leaves out.  No counterpart in the reference. */
+int64_t as_builder_scratch_bytes(as_builder *b, int64_t sub);
 /* executor.hpp:12 part_execute_code_builder: run only the listed sub-matrices (n_ids = 0: all), `repeat` launches,
  * synchronising after each; repeat = 0 takes the reference's own count, 185.2e9 / (padded elements of the listed
  * sub-matrices), at least 2 (executor.cc:247-255).  Returns 0 and (time_ms for all launches, gflops), <0 on
@@ -377,6 +406,10 @@ void as_search_free(as_search_result *r);
 const char *as_search_report(const as_search_result *r);
 /* everything upstream prints while searching + "gflops:/time:" + report + "finish search" */
 const char *as_search_log(const as_search_result *r);
+/* The best graph as numbers, in the layout as_graph_report takes (dense nodes, then per sub-matrix its nodes and
+ * its kernel node); returns how many numbers there are.  What main.cc:644 keeps as
+ * dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_t best_graph. */
+int64_t as_search_best_graph(const as_search_result *r, long *desc, uint64_t cap);
 /* out = {gflops, time_ms, candidates, failed candidates, seconds, seconds to best, sub-matrices, dense strategy} */
 int as_search_stats(const as_search_result *r, double out[8]);
 /* whilte_list_path_impl.cc:5318 execute_dense_view_matrix_and_compressed_sub_block_exe_graph_and_template:
@@ -395,6 +428,15 @@ int64_t as_strategy_report(int strategy, const long p[4], char *out, uint64_t ca
 /* exe_graph.cc:3317 convert_template_node_to_string of one kernel node */
 int64_t as_template_node_report(int template_type, long tblock_num, long thread_num_in_block, long thread_num_of_row_reduce,
                                 char *out, uint64_t cap);
+/* whilte_list_path_impl.cc:4150-4228 convert_dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_to_string_safety
+ * of a whole operator graph: the text as_search_report returns for a search's best graph, here for a graph given
+ * as numbers.  desc = n_dense, n_dense x (strategy, p0..p3), n_sub, then per sub-matrix: n_nodes, n_nodes x
+ * (strategy, p0..p3), template type, tblock_num, thread_num_in_block, thread_num_of_row_reduce; the knobs of the
+ * input node (DENSE_BEGIN_MEMORY_CACHE_INPUT_FILE_DIRECT) are element count, value type, largest column index,
+ * largest row index.  with_frame != 0: with the lines main.cc:646-657 prints around it ("gflops:", "time:", the
+ * graph and an empty line or "error", "finish search"), which is the tail of as_search_log.  Returns the text length. */
+int64_t as_graph_report(const long *desc, int64_t n_desc, int with_frame, float gflops, float time_ms, char *out,
+                        uint64_t cap);
 
 /* =====================================================================================
  * Thin HIP layer: what upstream reaches through system("./make_template.sh") (nvcc) and
@@ -432,6 +474,14 @@ int as_hip_event_record(void *ev, void *stream);
 int as_hip_event_sync(void *ev);
 int as_hip_event_elapsed_ms(void *start, void *stop, float *ms);
 int as_hip_stream_wait_event(void *stream, void *ev);
+/* stream capture into an executable graph and its replay (hipStreamBeginCapture / EndCapture / hipGraphInstantiate /
+ * hipGraphLaunch): for callers that replay a fixed launch sequence; no counterpart in the reference */
+int as_hip_graph_capture_begin(void *stream);
+int as_hip_graph_capture_end(void *stream, void **graph_exec);
+int as_hip_graph_launch(void *graph_exec, void *stream);
+int as_hip_graph_destroy(void *graph_exec);
+/* free and total device memory of the current GPU (hipMemGetInfo) */
+int as_hip_mem_info(uint64_t *free_bytes, uint64_t *total_bytes);
 int as_hip_launch(void *fn, unsigned grid, unsigned block, unsigned lds_bytes, void *stream, void **args);
 
 #ifdef __cplusplus

@@ -12,6 +12,7 @@
 
 #include <cstring>
 #include <iostream>
+#include <sstream>
 #include <vector>
 
 #include "exe_graph.hpp"
@@ -150,6 +151,13 @@ int ref_execute_node(void *hv, int node_type, int64_t sub, const long *scalars, 
       return 0;
     }
     case DENSE_ROW_DIV: {
+      // scalars {sub-block, strip height} and no list: strips of equal height inside a sub-block of an already
+      // divided matrix, fixed_len_row_div(matrix, sub_block, len) (op_manager.cc:243-365; upstream's var_len_row_div
+      // stops at a sub-block, :520)
+      if (n_list == 0 && n_scalars >= 2) {
+        fixed_len_row_div(h->m, h->m->block_coor_table.item_arr[scalars[0]], (int)scalars[1]);
+        return 0;
+      }
       vector<unsigned long> pos(list, list + n_list);
       if (pos.size() <= 2) return 0;
       var_len_row_div(h->m, NULL, pos);
@@ -159,8 +167,9 @@ int ref_execute_node(void *hv, int node_type, int64_t sub, const long *scalars, 
       if (n_list == 0) total_dense_block_sort(h->op);
       else total_dense_block_sort(h->op, vector<unsigned long>(list, list + n_list));
       return 0;
-    case DENSE_FIXED_COL_DIV:
-      fixed_len_col_div(h->m, NULL, (int)scalars[0]);
+    case DENSE_FIXED_COL_DIV:  // exe_graph.cc:1615-1640: the whole matrix first, a sub-block of the table afterwards
+      if (h->m->block_coor_table.item_arr.size() == 0) fixed_len_col_div(h->m, NULL, (int)scalars[0]);
+      else fixed_len_col_div(h->m, h->m->block_coor_table.item_arr[n_scalars >= 2 ? scalars[1] : 0], (int)scalars[0]);
       return 0;
     case COMPRESS:
       compress_dense_view(h->m);
@@ -743,6 +752,114 @@ int64_t ref_template_node_report(int type, long tblock_num, long thread_num_in_b
     default: node.template_param = two;
   }
   return put_text(convert_template_node_to_string(&node), out, cap);
+}
+
+}  // extern "C"
+
+// ---- the assembled report of a whole graph ------------------------------------------------------
+namespace {
+// a strategy with its knobs as the upstream parameter struct (heap: the graph keeps pointers; a test process ends soon)
+struct StrategyParam { exe_node_type node; void *param; };
+StrategyParam strategy_param(int strategy, const long *p) {
+  switch ((exe_node_param_set_strategy)strategy) {
+    case COMPRESSED_ROW_PADDING_DIRECT_PARAM_STRATEGY: { auto *s = new compressed_row_padding_direct_param_strategy_t(); s->multiply = p[0]; s->padding_row_length = p[1]; return {COMPRESSED_ROW_PADDING, s}; }
+    case COMPRESSED_TBLOCK_LEVEL_ROW_DIV_EVENLY_PARAM_STRATEGY: { auto *s = new compressed_tblock_level_row_div_evenly_param_strategy_t(); s->block_row_num = p[0]; return {COMPRESSED_TBLOCK_LEVEL_ROW_DIV, s}; }
+    case COMPRESSED_TBLOCK_LEVEL_ROW_DIV_ACC_TO_LEAST_NNZ_PARAM_STRATEGY: { auto *s = new compressed_tblock_level_row_div_acc_to_least_nnz_param_strategy_t(); s->nnz_low_bound = p[0]; return {COMPRESSED_TBLOCK_LEVEL_ROW_DIV, s}; }
+    case COMPRESSED_TBLOCK_LEVEL_COL_DIV_FIXED_PARAM_STRATEGY: { auto *s = new compressed_tblock_level_col_div_fixed_param_strategy_t(); s->col_block_nnz_num = p[0]; return {COMPRESSED_TBLOCK_LEVEL_COL_DIV, s}; }
+    case COMPRESSED_WARP_LEVEL_ROW_DIV_EVENLY_PARAM_STRATEGY: { auto *s = new compressed_warp_level_row_div_evenly_param_strategy_t(); s->warp_row_num_of_each_BLB = p[0]; return {COMPRESSED_WARP_LEVEL_ROW_DIV, s}; }
+    case COMPRESSED_WARP_LEVEL_COL_DIV_FIXED_PARAM_STRATEGY: { auto *s = new compressed_warp_level_col_div_fixed_param_strategy_t(); s->col_block_nnz_num = p[0]; return {COMPRESSED_WARP_LEVEL_COL_DIV, s}; }
+    case COMPRESSED_THREAD_LEVEL_ROW_DIV_NONE_PARAM_STRATEGY: return {COMPRESSED_THREAD_LEVEL_ROW_DIV, new compressed_thread_level_row_div_none_param_strategy_t()};
+    case COMPRESSED_THREAD_LEVEL_COL_DIV_FIXED_PARAM_STRATEGY: { auto *s = new compressed_thread_level_col_div_fixed_param_strategy_t(); s->col_block_nnz_num = p[0]; return {COMPRESSED_THREAD_LEVEL_COL_DIV, s}; }
+    case COMPRESSED_THREAD_LEVEL_NNZ_DIV_DIRECT_PARAM_STRATEGY: { auto *s = new compressed_thread_level_nnz_div_direct_param_strategy_t(); s->block_nnz_num = p[0]; return {COMPRESSED_THREAD_LEVEL_NNZ_DIV, s}; }
+    case DENSE_ROW_COARSE_SORT_FIXED_PARAM_STRATEGY: { auto *s = new dense_row_coarse_sort_fixed_param_strategy_t(); s->row_nnz_low_bound_step_size = p[0]; return {DENSE_ROW_COARSE_SORT, s}; }
+    case COMPRESS_NONE_PARAM_STRATEGY: return {COMPRESS, new compress_none_param_strategy_t()};
+    case DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ_PARAM_STRATEGY: {
+      auto *s = new dense_row_div_acc_to_exponential_increase_row_nnz_param_strategy_t();
+      s->lowest_nnz_bound_of_row = p[0]; s->highest_nnz_bound_of_row = p[1]; s->expansion_rate = p[2]; s->sub_dense_block_id = p[3];
+      return {DENSE_ROW_DIV, s};
+    }
+    case DENSE_BEGIN_MEMORY_CACHE_INPUT_FILE_DIRECT_PARAM_STRATEGY: {
+      // knobs: element count, value type, largest column index, largest row index; the elements themselves are
+      // placeholders (row i % rows, column i % cols, value 1), the report prints only those four
+      auto *s = new dense_begin_memory_cache_input_file_direct_param_strategy_t();
+      s->val_data_type = (data_type)p[1];
+      s->col_index_max = (unsigned long)p[2];
+      s->row_index_max = (unsigned long)p[3];
+      for (long i = 0; i < p[0]; i++) {
+        s->row_index_cache.push_back((unsigned long)i % (s->row_index_max + 1));
+        s->col_index_cache.push_back((unsigned long)i % (s->col_index_max + 1));
+        if (s->val_data_type == DOUBLE) s->double_val_cache.push_back(1.0); else s->float_val_cache.push_back(1.0f);
+      }
+      return {BEGIN_MEMORY_CACHE_INPUT_FILE, s};
+    }
+    default: return {COMPRESS, NULL};
+  }
+}
+}  // namespace
+
+extern "C" {
+
+// The report of a whole operator graph, assembled by upstream's own functions: the graph is built with
+// add_a_exe_node_and_param_strategy_to_exe_dense_sub_graph / ..._compressed_sub_graph (default_auto_tuner.cc:2131, 2281),
+// every sub-matrix gets its template node, and the text is what
+// convert_dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_to_string_safety
+// (whilte_list_path_impl.cc:4150-4228) returns.  `desc` = n_dense, n_dense x (strategy, p0..p3), n_sub, then per
+// sub-matrix: n_nodes, n_nodes x (strategy, p0..p3), template type, tblock_num, thread_num_in_block,
+// thread_num_of_row_reduce.  with_frame != 0: the text main.cc:646-657 prints around it (the same stream
+// insertions on the same float values) up to and including "finish search".
+int64_t ref_graph_report(const long *desc, int64_t n_desc, int with_frame, float gflops, float time_ms, char *out, uint64_t cap) {
+  std::string text;
+  {
+    Quiet q;
+    int64_t at = 0;
+    dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_t graph;
+    exe_dense_sub_graph_t &dense = graph.dense_sub_graph_and_param_strategy.dense_sub_graph;
+    param_strategy_of_sub_graph_t &dense_strategy = graph.dense_sub_graph_and_param_strategy.dense_sub_graph_param_strategy;
+    long n_dense = desc[at++];
+    for (long i = 0; i < n_dense; i++, at += 5) {
+      StrategyParam sp = strategy_param((int)desc[at], desc + at + 1);
+      if (sp.param == NULL) return -1;
+      add_a_exe_node_and_param_strategy_to_exe_dense_sub_graph(&dense, &dense_strategy, sp.node, (exe_node_param_set_strategy)desc[at], sp.param);
+    }
+    long n_sub = desc[at++];
+    for (long s = 0; s < n_sub; s++) {
+      compressed_sub_block_exe_graph_and_template_t sub;
+      long n_nodes = desc[at++];
+      for (long i = 0; i < n_nodes; i++, at += 5) {
+        StrategyParam sp = strategy_param((int)desc[at], desc + at + 1);
+        if (sp.param == NULL) return -1;
+        add_a_exe_node_and_param_strategy_to_exe_compressed_sub_graph(&sub.sub_graph, &sub.sub_graph_param_strategy, sp.node, (exe_node_param_set_strategy)desc[at], sp.param);
+      }
+      sub.temp_node.type = (template_type)desc[at];
+      long tblock = desc[at + 1], threads = desc[at + 2], row_reduce = desc[at + 3];
+      at += 4;
+      switch (sub.temp_node.type) {
+        case DIRECT_ATOM_TEMPLATE: { auto *t = new direct_atom_template_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        case DIRECT_ATOM_TEMPLATE_WARP_COMPRESS: { auto *t = new direct_atom_template_warp_compress_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        case DIRECT_ATOM_TEMPLATE_WARP_BLOCK_COMPRESS: { auto *t = new direct_atom_template_warp_block_compress_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        case SHARED_MEMORY_TEMPLATE: { auto *t = new shared_memory_template_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; t->thread_num_of_row_reduce = row_reduce; sub.temp_node.template_param = t; break; }
+        case SHARED_MEMORY_TEMPLATE_WARP_COMPRESS: { auto *t = new shared_memory_template_warp_compress_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; t->thread_num_of_row_reduce = row_reduce; sub.temp_node.template_param = t; break; }
+        case SHARED_MEMORY_LONG_ROW_TEMPLATE: { auto *t = new shared_memory_long_row_template_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        case SHARED_MEMORY_TOTAL_WARP_REDUCE_TEMPLATE: { auto *t = new shared_memory_total_warp_reduce_template_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; t->thread_num_of_row_reduce = row_reduce; sub.temp_node.template_param = t; break; }
+        case DIRECT_ATOM_TOTAL_WARP_REDUCE_TEMPLATE: { auto *t = new direct_atom_total_warp_reduce_template_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        case UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE: { auto *t = new unaligned_warp_reduce_same_TLB_size_template_node_param_t(); t->tblock_num = tblock; t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        case UNALIGNED_WARP_REDUCE_SAME_TLB_SIZE_TEMPLATE_WITH_WARP_REDUCE: { auto *t = new unaligned_warp_reduce_same_TLB_size_template_with_warp_reduce_node_param_t(); t->thread_num_in_block = threads; sub.temp_node.template_param = t; break; }
+        default: return -1;
+      }
+      graph.compressed_sub_block_exe_graph_and_template_vec.push_back(sub);
+    }
+    if (at != n_desc) return -1;
+    text = convert_dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_to_string_safety(graph);
+  }
+  if (with_frame) {
+    std::ostringstream f;
+    f << "gflops:" << gflops << std::endl;
+    f << "time:" << time_ms << std::endl;
+    if (gflops != 0) f << text << std::endl; else f << "error" << std::endl;
+    f << "finish search" << std::endl;
+    text = f.str();
+  }
+  return put_text(text, out, cap);
 }
 
 }  // extern "C"

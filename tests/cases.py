@@ -38,6 +38,14 @@ COLDIV50 = [("node", K.DENSE_FIXED_COL_DIV, (50,))]
 FINE_SORT = [("node", K.DENSE_FINE_SORT, (), ())]
 BAND_SORT = [("node", K.DENSE_FINE_SORT, (), (0, 37, 90, 150))]
 
+# Division of an existing sub-block (node parameters: DENSE_ROW_DIV scalars = {sub-block, height of equal strips},
+# DENSE_FIXED_COL_DIV scalars = {band width, sub-block}); the parent leaves the table, its parts go to the end
+ROWSTRIPS_UNI = ("node", K.DENSE_ROW_DIV, (), (0, 48, 128))          # uni40: rows [0, 48) and [48, 128)
+ROWSTRIPS_PL = ("node", K.DENSE_ROW_DIV, (), (0, 64, 160))           # pl: rows [0, 64) and [64, 160)
+SUBDIV_COLS = [ROWSTRIPS_UNI, ("node", K.DENSE_FIXED_COL_DIV, (50, 0))]   # the first strip into bands of 50 columns
+SUBDIV_ROWS = [ROWSTRIPS_UNI, ("node", K.DENSE_ROW_DIV, (0, 20), ())]     # the first strip into strips of 20 rows
+SUBDIV_ROWS_PL = [ROWSTRIPS_PL, ("node", K.DENSE_ROW_DIV, (1, 30), ())]   # the second strip into strips of 30 rows
+
 # (case id, matrix, dense strategies, skeleton applied to every sub-matrix, skeleton knobs)
 FORMAT_CASES = [
     ("ell_uni", "uni8", [], "S5", {"wave": 32}),
@@ -75,6 +83,11 @@ FORMAT_CASES = [
     ("coldiv50_uni_wlbcol", "uni40", COLDIV50, "S4", {"c": 8}),
     ("coldiv64_uni_longrow", "uni40", COLDIV64, "S8", {"b": 32}),
     ("coldiv64_uni_s2", "uni40", COLDIV64, "S2", {"m": 32, "len": 1, "s": 3}),
+    # a sub-block of an already divided matrix divided again (fixed_len_col_div / fixed_len_row_div with a sub-block)
+    ("subdiv_cols_uni_ell", "uni40", SUBDIV_COLS, "S5", {"wave": 32}),
+    ("subdiv_cols_uni_csr5", "uni40", SUBDIV_COLS, "S9", {"t": 3}),
+    ("subdiv_rows_uni_sell", "uni40", SUBDIV_ROWS, "S1", {"m": 32}),
+    ("subdiv_rows_pl_csr5", "pl", SUBDIV_ROWS_PL, "S9", {"t": 3}),
     # total_dense_block_sort: all rows by length (stable), and inside bands of rows
     ("finesort_pl_sell", "pl", FINE_SORT, "S1", {"m": 32}),
     ("finesort_irr_ell", "irr", FINE_SORT, "S5", {"wave": 32}),
@@ -106,6 +119,8 @@ EXTENSION_CASES = [
     ("tile_fem", "fem", [], "T1", {"slice": 32, "group": 16, "b": 256}),
     ("tile_irr_d3", "irr", D3, "T1", {"slice": 64, "group": 64, "b": 32}),
     ("tile_steps_d2", "steps", D2, "T1", {"slice": 4096, "group": 4096, "b": 8192}),
+    ("tile_subdiv_rows_pl", "pl", SUBDIV_ROWS_PL, "T1", {"slice": 64, "group": 16, "b": 100}),
+    ("tile_subdiv_cols_uni", "uni40", SUBDIV_COLS, "T1", {"slice": 32, "group": 16, "b": 64}),
     ("bin_pl_long", "pl_long", [], "T2", {"slice": 128, "group": 8, "b": 64}),
     ("bin_pl_sorted", "pl", SORT, "T2", {"slice": 64, "group": 32, "b": 100}),
     ("bin_fem", "fem", [], "T2", {"slice": 32, "group": 16, "b": 256}),

@@ -25,6 +25,8 @@ def main():
         "stop_rule": [H.stop_rule(L, "ref_", s, g) for s, g in H.STOP_CASES],
         "strategy_report": [H.strategy_report(L, "ref_", s, p) for s, p in H.STRATEGY_CASES],
         "template_node_report": [H.template_node_report(L, "ref_", *c) for c in H.TEMPLATE_NODE_CASES],
+        "graph_report": [H.graph_report(L, "ref_", *g) for g in H.GRAPH_CASES],
+        "graph_report_framed": [[H.graph_report(L, "ref_", *g, frame=f) for f in H.FRAME_CASES] for g in H.GRAPH_CASES[:2]],
     }
     path = os.path.join(HERE, "search_control.json")
     with open(path, "w") as f:

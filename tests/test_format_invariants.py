@@ -545,47 +545,129 @@ def test_tile_template_in_column_run_form(vdt, chunk, sort):
     assert not b.set_column_runs(0)
 
 
-def _emulate_product_bin_template(t, slice_width, group, sub_rows, x):
-    """y of the product-bin template's arrays: pass 1 writes val * x[slice base + column] of every element of every
-    trip to the element's position in row-group order, pass 2 adds the products of each row group's stream."""
+def _matrix_with_a_strip_of_zeros():
+    """200 rows of 8 elements with values, then 100 rows of one explicit zero; sorted and cut at row length 2."""
+    rng = np.random.default_rng(2)
+    lens = np.r_[np.full(200, 8), np.full(100, 1)]
+    r = np.repeat(np.arange(300), lens)
+    c = np.concatenate([np.sort(rng.choice(300, n, replace=False)) for n in lens])
+    v = np.where(r < 200, rng.uniform(0.5, 1.5, len(r)), 0.0)
+    m = A.Matrix.from_coo(300, 300, r, c, v, K.DOUBLE, wave=64)
+    m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+    m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (2, 2, 2, 0))
+    m.execute_strategy(K.COMPRESS_NONE)
+    assert m.info()["n_sub"] == 2
+    return m, r, c, v, rng.uniform(-1, 1, 300)
+
+
+def test_empty_template_takes_a_sub_matrix_of_zeros_and_has_no_kernel():
+    """EMPTY_TEMPLATE (upstream empty_op.cc): no arrays, no kernel text beyond a comment, and the builder clears y
+    because nobody else writes the rows of that sub-matrix.  A sub-matrix with a value is refused."""
+    from alphasparse_amd import skeletons as SK
+    m, r, c, v, x = _matrix_with_a_strip_of_zeros()
+    for sub in (0, 1):
+        SK.apply_skeleton(m, sub, "S1", m=64)
+    assert A.template_is_supported(m, 1, K.EMPTY_TEMPLATE) and not A.template_is_supported(m, 0, K.EMPTY_TEMPLATE)
+    b = A.Builder(m)
+    b.set_template(0, K.DIRECT_ATOM_TEMPLATE_WARP_COMPRESS)
+    b.set_template(1, K.EMPTY_TEMPLATE)
+    src = b.kernel_source()
+    assert "spmv_0(" in src and "spmv_1" not in src and "sub-matrix 1: no kernel" in src
+    assert b.clears_y()
+    b.compile()
+    with pytest.raises(K.AlphaSparseError, match="not empty"):
+        b.set_template(0, K.EMPTY_TEMPLATE)
+
+
+def test_row_ownership_asks_for_a_cleared_y_when_a_row_group_holds_no_element():
+    """Under row ownership the workgroup of a row group stores the group's rows at the end of its runs; a row group
+    without elements has no run, so nobody stores its rows and y must be cleared first."""
+    from alphasparse_amd import skeletons as SK
+    rows, cols, r, c, v, x = S.fem_blocks(3000, 27, 400)
+    for emptied, expect in (((750, 1000), 1), ((750, 999), 0), ((0, 0), 0)):
+        keep = (np.asarray(r) < emptied[0]) | (np.asarray(r) >= emptied[1])
+        m = A.Matrix.from_coo(rows, cols, r[keep], c[keep], v[keep].astype(np.float64), K.DOUBLE, wave=64)
+        m.execute_strategy(K.COMPRESS_NONE)
+        b = A.Builder(m)
+        b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=4000, group=250, b=4096)[0])
+        assert b.set_row_ownership(0)
+        assert b.describe(0)["row_groups_without_elements"] == expect and b.clears_y() == bool(expect)
+
+
+def _emulate_product_bin_template(t, slice_width, band_height, x, rows_of_y):
+    """y of the product-bin template's arrays, walked the way its two kernels walk them: pass 1 writes
+    val * x[slice base + column] of every element of every trip to the element's position in band order; pass 2 drops
+    the products of each band into the band's slots (the j-th element of the row of rank r at first[j] + r), adds up
+    every rank's slots and stores the sums to the band's rows of y.  Rows of y that the strip does not write stay NaN."""
     arr = {k: np.asarray(a[0]).astype(np.int64) for k, a in t["arrays"].items()}
+    sc = t["scalars"]
     val = np.asarray(t["val_arr"][0] if isinstance(t["val_arr"], tuple) else t["val_arr"], np.float64)
-    gs, gfu, pos, sfu, slot, yrow, lcol, width, sfr = (arr["group_slice"], arr["group_first_unit"], arr["product_position"],
-                                                       arr["sum_group_first_unit"], arr["slot_in_group"], arr["y_row_index"],
-                                                       arr["col_index_arr"], arr["sum_group_width"], arr["sum_group_first_row"])
-    assert len(gfu) == len(gs) + 1 and gfu[0] == 0 and gfu[-1] * 256 == len(val) == len(lcol) == len(pos)
+    gs, gfu, ufb, shift, lcol = arr["group_slice"], arr["group_first_unit"], arr["unit_first_bin"], arr["bin_shift"], arr["col_index_arr"]
+    bfu, bfc, yb, cnt, slot = (arr["band_first_unit"], arr["band_first_count"], arr["band_y_begin"], arr["band_slot_count"],
+                               arr["slot_in_band"])
+    flag, lcol = lcol >> 15, lcol & 0x7fff
+    assert len(gfu) == len(gs) + 1 and gfu[0] == 0 and gfu[-1] * 256 == len(val) == len(lcol)
     assert (np.diff(gfu) > 0).all() and (np.diff(gs) >= 0).all() and (lcol < slice_width).all()
-    # summing groups: consecutive rows, never across a row group of the division, slots within the budget
-    # (2048 slots for a strip this small) unless a single row needs more
-    nsum = len(width)
-    assert len(sfr) == len(sfu) == nsum + 1 and sfr[0] == 0 and sfr[-1] == sub_rows and (np.diff(sfr) > 0).all()
-    assert sfu[0] == 0 and sfu[-1] * 256 == len(slot) and (np.diff(sfu) >= 0).all()
-    assert (sfr[:-1] // group == (sfr[1:] - 1) // group).all()
-    n_rows = np.diff(sfr)
-    assert (n_rows * width + 1 <= t["scalars"]["max_slots"]).all() and t["scalars"]["max_slots"] <= 2048
-    # real elements go to distinct places inside the product stream, padding to the spare slot behind it
-    real = pos < len(slot)
-    assert len(np.unique(pos[real])) == real.sum() and (pos[~real] == len(slot)).all() and (val[~real] == 0).all()
-    product = np.zeros(len(slot) + 1)
-    written = np.zeros(len(slot) + 1, bool)
+    nband = sc["band_num"]
+    assert len(bfu) == len(bfc) == nband + 1 == len(yb) + 1 and bfu[0] == 0 and bfu[-1] * 256 == len(slot) == sc["product_len"]
+    # a unit knows how many bins start before it; the first element of every slice opens one
+    assert len(ufb) == gfu[-1] + 1 and ufb[-1] == len(shift) == flag.sum()
+    assert (ufb[:-1] == np.concatenate([[0], np.cumsum(flag)])[:-1:256]).all()
+    product = np.zeros(len(slot) + 256)
+    written = np.zeros(len(slot) + 256, bool)
     for trip in range(len(gs)):
         k0, k1 = gfu[trip] * 256, gfu[trip + 1] * 256
+        assert flag[k0] == 1 or (trip > 0 and gs[trip - 1] == gs[trip])      # a slice starts with a new bin
         xs = np.zeros(slice_width)
         part = x[gs[trip] * slice_width:(gs[trip] + 1) * slice_width]
         xs[:len(part)] = part
-        product[pos[k0:k1]] = val[k0:k1] * xs[lcol[k0:k1]]
-        written[pos[k0:k1]] = True
-    y = np.zeros(int(yrow.max()) + 1)
-    for g in range(nsum):
-        k0, k1 = sfu[g] * 256, sfu[g + 1] * 256
-        live = n_rows[g]
-        slots = np.zeros(width[g] * live + 1)
+        bin0 = ufb[gfu[trip]] - 1 if ufb[gfu[trip]] else 0
+        in_lds = shift[bin0:ufb[gfu[trip + 1]]]                              # the shifts the trip keeps in LDS
+        assert 1 <= len(in_lds) <= sc["max_trip_bins"] <= 4096
+        for u in range(gfu[trip], gfu[trip + 1]):                            # a wavefront step
+            k = np.arange(u * 256, (u + 1) * 256)
+            local = ufb[u] - bin0 - 1 + np.cumsum(flag[k])                   # flags up to and including the element
+            assert (local >= 0).all()
+            place = (k + in_lds[local]) & 0xffffffff
+            assert not written[place[place < len(slot)]].any() and (val[k][place >= len(slot)] == 0).all()
+            product[place] = val[k] * xs[lcol[k]]
+            written[place] = True
+    # padding of the first pass (value 0) lands behind the products
+    assert (product[len(slot):] == 0).all()
+    written, product = written[:len(slot) + 1], product[:len(slot) + 1]
+    y = np.full(rows_of_y, np.nan)
+    stored = np.zeros(rows_of_y, int)
+    for g in range(nband):
+        first = cnt[bfc[g]:bfc[g + 1]]                 # first[j]: slots of the elements 0..j-1 of all rows
+        width = len(first) - 1
+        assert width >= 1 and first[0] == 0 and (np.diff(first) >= 0).all() and (np.diff(first, 2) <= 0).all()
+        assert width <= sc["max_width"] and first[-1] + 1 <= sc["max_slots"]
+        k0, k1 = bfu[g] * 256, bfu[g + 1] * 256
+        assert k1 - k0 >= first[-1] > k1 - k0 - 256 or (first[-1] == 0 and k1 == k0)
+        slots = np.full(first[-1] + 1, np.nan)
         real_slot = slot[k0:k1][written[k0:k1]]
-        assert (slot[k0:k1][~written[k0:k1]] == width[g] * live).all()   # group padding: spare slot, never written
-        assert len(np.unique(real_slot)) == len(real_slot) and (real_slot < width[g] * live).all()
-        slots[slot[k0:k1]] = product[k0:k1]
+        assert (slot[k0:k1][~written[k0:k1]] == first[-1]).all()      # band padding: spare slot, never written
+        assert sorted(real_slot) == list(range(first[-1]))            # every slot filled exactly once: no clear needed
         assert (product[k0:k1][~written[k0:k1]] == 0).all()
-        y[yrow[sfr[g]:sfr[g] + live]] = slots[:width[g] * live].reshape(width[g], live).sum(0)
+        slots[slot[k0:k1]] = product[k0:k1]
+        live = first[1]
+
+        def row_sum(r):
+            return sum(slots[first[j] + r] for j in range(width) if r < first[j + 1] - first[j])
+        if sc["dense_y"]:
+            ye, rank = arr["band_y_end"], arr["rank_of_y_row"]
+            assert yb[g] < ye[g] <= yb[g] + band_height and (g == 0 or ye[g - 1] <= yb[g])
+            for p in range(yb[g], ye[g]):
+                if rank[p] != 0xffff:
+                    y[sc["y_base"] + p] = row_sum(rank[p]) if rank[p] < live else 0.0
+                    stored[sc["y_base"] + p] += 1
+        else:
+            bfr, place = arr["band_first_row"], arr["y_row_of_rank"]
+            assert live <= bfr[g + 1] - bfr[g] and (place[bfr[g]:bfr[g + 1]] < band_height).all()
+            for r in range(bfr[g + 1] - bfr[g]):
+                y[sc["y_base"] + yb[g] + place[bfr[g] + r]] = row_sum(r)
+                stored[sc["y_base"] + yb[g] + place[bfr[g] + r]] += 1
+    assert stored.max() == 1 and stored.sum() == sc["sub_rows"]
     return y
 
 
@@ -593,7 +675,7 @@ def _emulate_product_bin_template(t, slice_width, group, sub_rows, x):
                                                           (64, 4096, 4096, True)])
 def test_product_bin_template(slice_width, group, blb, sort):
     """SHARED_MEMORY_PRODUCT_BIN_TEMPLATE on the tile division: slices padded to whole 256-element units, trips cut
-    inside slices, bins = (row group, slice) pieces of the element stream; two passes reproduce y = A x."""
+    inside slices, bands of `group` rows of y with their rows ranked by falling length; two passes reproduce y = A x."""
     from alphasparse_amd import skeletons as SK
     rows, cols, r, c, v, x = cases._steps([3] * 40 + [9] * 24 + [1] * 30 + [2] * 70 + [7] * 13, 640, 22)
     m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.FLOAT, wave=64)
@@ -609,49 +691,101 @@ def test_product_bin_template(slice_width, group, blb, sort):
     b = A.Builder(m)
     b.set_template(0, tp, compress=False)
     t = b.template_dump(0)
-    y = _emulate_product_bin_template(t, slice_width, group, rows, x.astype(np.float64))
+    assert t["scalars"]["dense_y"] == 1 and t["scalars"]["band_num"] == -(-rows // group)
+    y = _emulate_product_bin_template(t, slice_width, group, x.astype(np.float64), rows)
     assert np.allclose(y, yref, rtol=1e-12, atol=1e-12)
-    assert t["arrays"]["col_index_arr"][1] == "UNSIGNED_SHORT" and t["arrays"]["slot_in_group"][1] == "UNSIGNED_SHORT"
+    assert t["arrays"]["col_index_arr"][1] == "UNSIGNED_SHORT" and t["arrays"]["slot_in_band"][1] == "UNSIGNED_SHORT"
+    assert t["arrays"]["rank_of_y_row"][1] == "UNSIGNED_SHORT"
     b.set_template(0, tp, compress=True)
     src = b.kernel_source()
-    assert "spmv_0_finish" in src and "scratch_arr" in src and ("y_row_index[" in src) == sort
+    assert "spmv_0_finish" in src and "scratch_arr" in src and "rank_of_y_row[" in src
+    assert not b.clears_y()     # the second pass stores every row of the strip
+
+
+def _short_rows_with_a_few_longer(rows, seed, longer=50):
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(1, 4, rows)
+    lens[rng.choice(rows, longer, replace=False)] = rng.integers(5, 30, longer)
+    r = np.repeat(np.arange(rows), lens)
+    c = np.concatenate([np.sort(rng.choice(rows, n, replace=False)) for n in lens])
+    return lens, r, c, rng.uniform(-1, 1, len(r)), rng.uniform(-1, 1, rows)
 
 
 def test_product_bin_template_takes_sorted_rows_band_by_band():
-    """Under a sort the product-bin template keeps the rows longer than 4 elements in front and orders the others by
-    bands of 4096 rows of y and only inside a band by length: a summing group stays inside one band, and the two
-    passes still reproduce y = A x."""
+    """Under a sort the product-bin template still takes the rows band by band of y (here 4096 rows of y each) and
+    ranks them by falling length inside a band, whatever their place in the sorted strip: the ranks of a band are a
+    permutation of its rows, a longer row never has a higher rank than a shorter one, and the two passes reproduce
+    y = A x."""
     from alphasparse_amd import skeletons as SK
-    rng = np.random.default_rng(3)
     rows = cols = 10000
-    lens = rng.integers(1, 4, rows)
-    lens[rng.choice(rows, 50, replace=False)] = rng.integers(5, 30, 50)   # a few rows too long for the bands
-    r = np.repeat(np.arange(rows), lens)
-    c = np.concatenate([np.sort(rng.choice(cols, n, replace=False)) for n in lens])
-    v = rng.uniform(-1, 1, len(r))
-    x = rng.uniform(-1, 1, cols)
+    lens, r, c, v, x = _short_rows_with_a_few_longer(rows, 3)
     m = A.Matrix.from_coo(rows, cols, r, c, v, K.DOUBLE, wave=64)
     m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
     m.execute_strategy(K.COMPRESS_NONE)
-    tp = SK.apply_skeleton(m, 0, "T2", slice=1024, group=8192, b=4096)[0]
+    tp = SK.apply_skeleton(m, 0, "T2", slice=1024, group=4096, b=4096)[0]
     b = A.Builder(m)
     b.set_template(0, tp, compress=False)
     t = b.template_dump(0)
-    yrow = np.asarray(t["arrays"]["y_row_index"][0]).astype(np.int64)
-    sfr = np.asarray(t["arrays"]["sum_group_first_row"][0]).astype(np.int64)
-    assert sorted(yrow) == list(range(rows))
-    length = np.bincount(r, minlength=rows)[yrow]
-    assert (length[:50] > 4).all() and (np.diff(length[:50]) <= 0).all() and (length[50:] <= 4).all()  # long rows in front
-    assert (np.diff(yrow[50:] // 4096) >= 0).all()                # then band by band
-    for band in range(3):
-        inside = length[50:][yrow[50:] // 4096 == band]
-        assert (np.diff(inside) <= 0).all()                       # longest first inside a band
-    for g in range(len(sfr) - 1):
-        assert sfr[g + 1] <= 50 or (sfr[g] >= 50 and len(set(yrow[sfr[g]:sfr[g + 1]] // 4096)) == 1)   # a summing group stays in its band
+    assert t["scalars"]["band_num"] == 3 and t["scalars"]["dense_y"] == 1 and t["scalars"]["y_base"] == 0
+    rank = np.asarray(t["arrays"]["rank_of_y_row"][0]).astype(np.int64)
+    yb, ye = (np.asarray(t["arrays"][k][0]).astype(np.int64) for k in ("band_y_begin", "band_y_end"))
+    assert list(yb) == [0, 4096, 8192] and list(ye) == [4096, 8192, 10000]
+    for g in range(3):
+        inside = rank[yb[g]:ye[g]]
+        assert sorted(inside) == list(range(ye[g] - yb[g]))
+        by_rank = lens[yb[g]:ye[g]][np.argsort(inside)]
+        assert (np.diff(by_rank) <= 0).all()                          # longest first
+        same = np.flatnonzero(np.diff(by_rank) == 0)
+        assert (np.diff(np.argsort(inside))[same] > 0).all()          # rows of equal length in the order of y
     yref = np.zeros(rows)
     np.add.at(yref, r, v * x[c])
-    y = _emulate_product_bin_template(t, 1024, 8192, rows, x)
+    y = _emulate_product_bin_template(t, 1024, 4096, x, rows)
     assert np.allclose(y, yref, rtol=1e-12, atol=1e-12)
+
+
+def test_product_bin_template_cuts_bands_by_their_lds_slots_and_stores_by_rank_in_a_thin_strip():
+    """A band ends where its elements would no longer fit its LDS slots (80 KB: 10239 fp64 elements), and a strip
+    that holds few of the rows of y it spans (here the rows of 5 or more elements of a sorted matrix) keeps a 16-bit
+    place in y per rank instead of a rank per row of y."""
+    from alphasparse_amd import skeletons as SK
+    rows = cols = 12000
+    rng = np.random.default_rng(8)
+    lens = np.full(rows, 7)
+    r = np.repeat(np.arange(rows), lens)
+    c = np.concatenate([np.sort(rng.choice(cols, n, replace=False)) for n in lens])
+    v, x = rng.uniform(-1, 1, len(r)), rng.uniform(-1, 1, cols)
+    m = A.Matrix.from_coo(rows, cols, r, c, v, K.DOUBLE, wave=64)
+    m.execute_strategy(K.COMPRESS_NONE)
+    tp = SK.apply_skeleton(m, 0, "T2", slice=4096, group=65536, b=4096)[0]
+    b = A.Builder(m)
+    b.set_template(0, tp, compress=False)
+    t = b.template_dump(0)
+    per_band = 10239 // 7
+    assert t["scalars"]["band_num"] == -(-rows // per_band) and t["scalars"]["max_slots"] == per_band * 7 + 1
+    yref = np.zeros(rows)
+    np.add.at(yref, r, v * x[c])
+    assert np.allclose(_emulate_product_bin_template(t, 4096, 65536, x, rows), yref, rtol=1e-12, atol=1e-12)
+    # the thin strip
+    rows = cols = 10000
+    lens, r, c, v, x = _short_rows_with_a_few_longer(rows, 5, longer=200)
+    m = A.Matrix.from_coo(rows, cols, r, c, v, K.DOUBLE, wave=64)
+    m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+    m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (5, 5, 2, 0))
+    m.execute_strategy(K.COMPRESS_NONE)
+    assert m.info()["n_sub"] == 2                      # sorted: the 200 rows of 5 or more elements come first
+    tp = SK.apply_skeleton(m, 0, "T2", slice=1024, group=2048, b=4096)[0]
+    b = A.Builder(m)
+    b.set_template(0, tp, compress=False)
+    t = b.template_dump(0)
+    assert t["scalars"]["sub_rows"] == 200
+    assert t["scalars"]["dense_y"] == 0 and "y_row_of_rank" in t["arrays"] and "rank_of_y_row" not in t["arrays"]
+    yref = np.zeros(rows)
+    np.add.at(yref, r, v * x[c])
+    y = _emulate_product_bin_template(t, 1024, 2048, x, rows)
+    mine = lens >= 5
+    assert np.isnan(y[~mine]).all() and np.allclose(y[mine], yref[mine], rtol=1e-12, atol=1e-12)
+    b.set_template(0, tp, compress=True)
+    assert "y_row_of_rank[" in b.kernel_source()
 
 
 def test_relative_columns_of_the_ell_template():

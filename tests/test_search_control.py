@@ -62,6 +62,31 @@ def test_template_node_report_matches_upstream(want, where):
         assert H.template_node_report(K.lib(), "as_", *case) == w, K.TEMPLATE_NAMES[case[0]]
 
 
+@EVERYWHERE
+def test_graph_report_matches_upstream(want, where):
+    """The assembled report of whole graphs (one to three strips, every dense strategy, nine template types),
+    byte for byte what upstream's own functions return for graphs built with upstream's own node adders; and with
+    the lines upstream's main prints around it."""
+    for g, w in zip(H.GRAPH_CASES, want["graph_report"]):
+        assert H.graph_report(K.lib(), "as_", *g) == w
+    for g, ws in zip(H.GRAPH_CASES[:2], want["graph_report_framed"]):
+        for f, w in zip(H.FRAME_CASES, ws):
+            assert H.graph_report(K.lib(), "as_", *g, frame=f) == w, f
+
+
+def test_graph_report_shape():
+    """Known answers that do not need the fixture: node order, sub_matrix_id lines, brace nesting of the kernel nodes."""
+    text = H.graph_report(K.lib(), "as_", *H.GRAPH_CASES[2])
+    assert text.startswith("{\nstrategy_type:DENSE_BEGIN_MEMORY_CACHE_INPUT_FILE_DIRECT_PARAM_STRATEGY\nnode_type:BEGIN_MEMORY_CACHE_INPUT_FILE\n"
+                           "{\nnnz:5000\ndata_type:DOUBLE\ncol_index_max:99999\nrow_index_max:49999\n}\n}\n")
+    assert text.count("sub_matrix_id:") == 2 and text.index("sub_matrix_id:0\n") < text.index("sub_matrix_id:1\n")
+    assert text.index("node_type:COMPRESS\n") < text.index("sub_matrix_id:0\n")
+    framed = H.graph_report(K.lib(), "as_", *H.GRAPH_CASES[0], frame=(0.0, 5.0))
+    assert framed == "gflops:0\ntime:5\nerror\nfinish search\n"
+    framed = H.graph_report(K.lib(), "as_", *H.GRAPH_CASES[0], frame=(12.5, 0.25))
+    assert framed == "gflops:12.5\ntime:0.25\n" + H.graph_report(K.lib(), "as_", *H.GRAPH_CASES[0]) + "\nfinish search\n"
+
+
 def test_live_upstream_on_random_inputs():
     import ref_lib
     if not ref_lib.available():
@@ -86,3 +111,12 @@ def test_live_upstream_on_random_inputs():
     for tp in range(10):
         args = (tp, int(rng.integers(1, 1 << 20)), 64 * int(rng.integers(1, 17)), int(2 ** rng.integers(0, 7)))
         assert H.template_node_report(L, "as_", *args) == H.template_node_report(R, "ref_", *args)
+    # whole graphs with random knobs and launch parameters
+    for dense, subs in H.GRAPH_CASES:
+        dense2 = [(s, tuple(int(x) for x in rng.integers(1, 5000, len(p))) if s != 10 else p) for s, p in dense]
+        subs2 = [([(s, tuple(int(x) for x in rng.integers(1, 5000, len(p)))) for s, p in nodes],
+                  (tpl[0], int(rng.integers(1, 1 << 20)), 64 * int(rng.integers(1, 17)), int(2 ** rng.integers(0, 7))))
+                 for nodes, tpl in subs]
+        frame = (float(np.float32(rng.gamma(2.0, 300.0))), float(np.float32(rng.gamma(2.0, 0.05))))
+        assert H.graph_report(L, "as_", dense2, subs2) == H.graph_report(R, "ref_", dense2, subs2)
+        assert H.graph_report(L, "as_", dense2, subs2, frame) == H.graph_report(R, "ref_", dense2, subs2, frame)

@@ -31,6 +31,20 @@ def _check_best(res, rows, r, c, v, x, gpu, npd):
     return b
 
 
+def _template_types(numbers):
+    """Template type of every sub-matrix in the flat description of a graph."""
+    at = 1 + 5 * numbers[0]
+    out = []
+    n_sub = numbers[at]
+    at += 1
+    for _ in range(n_sub):
+        at += 1 + 5 * numbers[at]
+        out.append(numbers[at])
+        at += 4
+    assert at == len(numbers)
+    return out
+
+
 CASES = {
     "laplacian": (lambda: S.laplacian_5pt(160), K.FLOAT),
     "power_law": (lambda: S.power_law(30000, max_len=5000, mean_len=14.0, seed=7), K.FLOAT),
@@ -56,6 +70,22 @@ def test_search_result_is_correct_and_reported(gpu, name):
     assert "node_type:COMPRESS\n" in rep
     log = res.log
     assert log.endswith("finish search\n") and ("gflops:%g\n" % res.gflops) in log
+    # the report is, byte for byte, what as_graph_report makes of the best graph's numbers, and the log ends with
+    # that text in the frame of upstream's main
+    import search_hooks as H
+    numbers = res.best_graph()
+    assert H.without_extra_keys(rep) == H.graph_report_of_numbers(K.lib(), "as_", numbers)
+    # ... and what upstream's own report function returns for the same graph built with upstream's own node adders
+    # (the compiled upstream code travels with the tree; without it the committed answers of
+    # tests/test_search_control.py pin the same functions)
+    import ref_lib
+    upstream_only = all(t < 10 for t in _template_types(numbers))
+    if ref_lib.available() and upstream_only:
+        want = H.graph_report_of_numbers(ref_lib.lib(), "ref_", numbers)
+        assert H.without_extra_keys(rep) == want, (rep, want)
+        framed = H.graph_report_of_numbers(ref_lib.lib(), "ref_", numbers, frame=(res.gflops, res.time_ms))
+        assert H.without_extra_keys(log).endswith(framed), (log[-len(framed) - 200:], framed)
+        print(name, "report equals upstream's text for the same graph (%d bytes)" % len(want), flush=True)
     b = _check_best(res, rows, r, c, v, x, gpu, NP[vdt])
     # executor entry points on the rebuilt graph
     ok, ms, gf = A.part_execute_code_builder(b, list(range(int(res.n_sub))), 20)

@@ -398,6 +398,37 @@ def test_tile_template_with_row_blocks(gpu, vdt, runs, threads):
         b.close()
 
 
+@pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("form", ["columns", "runs", "blocks"])
+def test_tile_template_under_row_ownership_with_a_row_group_without_elements(gpu, vdt, form):
+    """A row group that holds no element has no run under row ownership, so its owner never stores its rows: the
+    builder must clear y for such a graph.  Rows 756..1007 (one whole row group of 252 rows) of a banded block matrix
+    are emptied; y holds NaN before the call and must come back as A x with zeros in the emptied rows."""
+    rows, cols, r, c, v, x = S.fem_blocks(3000, 27, 400)
+    keep = (np.asarray(r) < 756) | (np.asarray(r) >= 1008)
+    r, c, v = r[keep], c[keep], v[keep]
+    npd = NP[vdt]
+    v, x = v.astype(npd), x.astype(npd)
+    y_ref, mag = oracle_y(rows, r, c, v, x)
+    assert (y_ref[756:1008] == 0).all()
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    m.execute_strategy(K.COMPRESS_NONE)
+    b = A.Builder(m)
+    b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=4000, group=252, b=4096)[0])
+    if form != "columns":
+        assert b.set_column_runs(0)
+    assert b.set_row_ownership(0)
+    if form == "blocks":
+        assert b.set_row_blocks(0, 3)
+    assert b.describe(0)["row_groups_without_elements"] == 1 and b.clears_y()
+    b.compile().upload(gpu)
+    print("case: row ownership, empty row group", form, vdt, flush=True)
+    y = b.spmv_device(x)
+    assert not np.isnan(y).any() and (y[756:1008] == 0).all()
+    assert_y(y, y_ref, mag, npd, "tile template, row ownership, a row group without elements")
+    b.close()
+
+
 @pytest.mark.parametrize("position", [K.END_PADDING, K.TOP_PADDING], ids=["end", "top"])
 @pytest.mark.parametrize("skel,kw", [("S5", {}), ("S1", {"m": 64}), ("T1", {"slice": 1024, "group": 512, "b": 2048})],
                          ids=["S5", "S1", "T1"])
@@ -681,6 +712,25 @@ def test_finish_of_a_tile_strip_carried_by_the_next_strips_kernel(gpu, vdt):
     assert b.finish_carrier(0) == 1 and "carried_sum" in src
     assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, rows already in sorted order")
     assert_y(b.spmv_device(z), *oracle_y(rows, r2, c2, v2, z), npd, "carried finish, rows already in sorted order, second call")
+    b.close()
+
+
+def test_empty_template_launches_nothing_and_leaves_zeros(gpu):
+    """A graph whose second strip holds only explicit zeros and has EMPTY_TEMPLATE: y = A x with zeros in the rows of
+    that strip, from a y full of NaN."""
+    from test_format_invariants import _matrix_with_a_strip_of_zeros
+    m, r, c, v, x = _matrix_with_a_strip_of_zeros()
+    for sub in (0, 1):
+        SK.apply_skeleton(m, sub, "S1", m=64)
+    b = A.Builder(m)
+    b.set_template(0, K.DIRECT_ATOM_TEMPLATE_WARP_COMPRESS)
+    b.set_template(1, K.EMPTY_TEMPLATE)
+    b.compile().upload(gpu)
+    y_ref, mag = oracle_y(300, r.astype(np.uint64), c.astype(np.uint64), v, x)
+    y = b.spmv_device(x)
+    assert (y[200:] == 0).all()
+    assert_y(y, y_ref, mag, np.float64, "EMPTY_TEMPLATE on the strip of zeros")
+    assert_y(b.spmv(x), y_ref, mag, np.float64, "EMPTY_TEMPLATE, host vectors")
     b.close()
 
 

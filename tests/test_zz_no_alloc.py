@@ -17,7 +17,7 @@ NP = {K.FLOAT: np.float32, K.DOUBLE: np.float64}
 STATIC_SCRATCH_BYTES = 64 << 20
 
 
-def _two_strip_builder(gpu, rows, max_len, seed, vdt):
+def _two_strip_builder(gpu, rows, max_len, seed, vdt, serial=True, carry=True):
     """Coarse sort, rows of 16 or more elements through the tile template (scratch: the strip's row sums, must start
     at zero), the others through the product-bin template (scratch: the products): the shape of the graphs the
     search returns for the power-law and the extremely irregular workloads."""
@@ -33,8 +33,10 @@ def _two_strip_builder(gpu, rows, max_len, seed, vdt):
     b = A.Builder(m)
     b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=1024, group=512, b=2048)[0])
     b.set_template(1, SK.apply_skeleton(m, 1, "T2", slice=1024, group=4096, b=2048)[0])
-    b.set_serial_launch(True)
+    b.set_serial_launch(serial)
+    b.set_finish_carry(carry)
     b.compile().upload(gpu)
+    b.coo = (rows, r, c, v)       # for callers that check other vectors x
     y_ref, mag = O.spmv_csr(O.coo_to_csr(rows, r), c.astype(np.uint32), v, x)
     return b, x, y_ref, mag, npd
 
@@ -45,11 +47,13 @@ def _check(y, y_ref, mag, npd, what):
 
 
 @pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
-def test_no_alloc_entry_point_matches_the_allocating_one(gpu, vdt):
-    big = _two_strip_builder(gpu, 20000, 3000, 31, vdt)
-    small = _two_strip_builder(gpu, 3000, 700, 32, vdt)
+@pytest.mark.parametrize("serial,carry", [(True, True), (True, False), (False, True)],
+                         ids=["serial_carried", "serial_own_finish", "concurrent_streams"])
+def test_no_alloc_entry_point_matches_the_allocating_one(gpu, vdt, serial, carry):
+    big = _two_strip_builder(gpu, 20000, 3000, 31, vdt, serial, carry)
+    small = _two_strip_builder(gpu, 3000, 700, 32, vdt, serial, carry)
     for name, (b, x, y_ref, mag, npd) in (("first call", big), ("second call, smaller matrix", small), ("third call", big)):
-        print("case: no-alloc", name, b.rows, flush=True)
+        print("case: no-alloc", name, b.rows, "serial" if serial else "concurrent", "carried" if carry else "own finish", flush=True)
         need = b.static_scratch_need()
         assert 0 < need <= STATIC_SCRATCH_BYTES
         y_alloc = b.spmv_device(x)
@@ -96,3 +100,75 @@ def test_no_alloc_entry_point_needs_an_uploaded_builder(gpu):
     with pytest.raises(K.AlphaSparseError, match="upload"):
         b.spmv_device(x, no_alloc=True)
     b.close()
+
+
+def test_no_alloc_call_leaves_device_memory_as_it_was(gpu):
+    """Free device memory (hipMemGetInfo) is the same before and after calls of the entry point that allocates
+    nothing, on buffers allocated beforehand."""
+    b, x, y_ref, mag, npd = _two_strip_builder(gpu, 20000, 3000, 31, K.DOUBLE)
+    dx, dy = A.DeviceArray(x), A.DeviceArray(np.full(b.rows, np.nan, npd))
+    b.spmv_device_async(dx, dy, None, no_alloc=True)       # first call: nothing left to set up afterwards
+    b.sync()
+    before = A.device_memory_free_bytes()
+    for _ in range(5):
+        b.spmv_device_async(dx, dy, None, no_alloc=True)
+    b.sync()
+    assert A.device_memory_free_bytes() == before
+    _check(dy.get(), y_ref, mag, npd, "no-alloc calls on buffers of the caller")
+    dx.free()
+    dy.free()
+    b.close()
+
+
+@pytest.mark.parametrize("vdt", [K.FLOAT, K.DOUBLE], ids=["fp32", "fp64"])
+def test_no_alloc_async_call_replayed_as_a_hip_graph(gpu, vdt):
+    """as_builder_spmv_device_no_alloc_async recorded by a stream capture (it allocates nothing, waits for nothing and
+    clears with fill kernels, not memset nodes) and replayed three times with a different x each time, the program's
+    own eager work and waits in between: every replay must give A x for the x of that replay.  Two graphs: the
+    two-strip graph (scratch of both strips in the static array, the tile strip's piece cleared by the fill kernel,
+    finish carried) and a graph that starts with a clear of y."""
+    npd = NP[vdt]
+    cases = [_two_strip_builder(gpu, 20000, 3000, 31, vdt)]
+    rows, cols, r, c, v, x = S.power_law(8000, max_len=900, mean_len=20.0, seed=5)
+    m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+    m.execute_strategy(K.COMPRESS_NONE)
+    bt = A.Builder(m)
+    bt.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=1024, group=512, b=2048)[0])
+    bt.compile().upload(gpu)
+    assert bt.clears_y()
+    bt.coo = (rows, r, c, v.astype(npd))
+    y_ref, mag = O.spmv_csr(O.coo_to_csr(rows, r), c.astype(np.uint32), v.astype(npd), x.astype(npd))
+    cases.append((bt, x.astype(npd), y_ref, mag, npd))
+    stream = A.Stream()
+    for which, (b, x, y_ref, mag, _) in enumerate(cases):
+        rows, r, c, v = b.coo
+        row_ptr, col32 = O.coo_to_csr(rows, r), np.asarray(c).astype(np.uint32)
+        dx, dy = A.DeviceArray(x), A.DeviceArray(np.full(b.rows, np.nan, npd))
+        b.spmv_device_async(dx, dy, stream, no_alloc=True)       # eager, before the capture
+        stream.sync()
+        _check(dy.get(), y_ref, mag, npd, "eager call before the capture")
+        print("case: capture", which, b.rows, vdt, flush=True)
+        stream.capture_begin()
+        b.spmv_device_async(dx, dy, stream, no_alloc=True)
+        graph = stream.capture_end()
+        rng = np.random.default_rng(11 + which)
+        for replay in range(3):
+            x2 = rng.uniform(-1, 1, b.cols).astype(npd)
+            dx.set(x2)
+            dy.set(np.full(b.rows, np.nan, npd))
+            stream.graph_launch(graph)
+            stream.sync()
+            y2 = dy.get()
+            y_want, mag2 = O.spmv_csr(row_ptr, col32, v, x2)
+            _check(y2, y_want, mag2, npd, "replay %d" % replay)
+            # eager work of the program between two replays: the allocating entry point on the same x
+            _check(b.spmv_device(x2), y_want, mag2, npd, "eager call between replays")
+        dx.set(x)                                                # and the first x once more, through the graph
+        stream.graph_launch(graph)
+        stream.sync()
+        _check(dy.get(), y_ref, mag, npd, "replay with the first x")
+        stream.graph_destroy(graph)
+        dx.free()
+        dy.free()
+        b.close()
+    stream.destroy()
