@@ -42,6 +42,8 @@ def _bind(L):
     L.as_builder_set_serial_launch.argtypes = [vp, C.c_int]
     L.as_builder_set_finish_carry.argtypes = [vp, C.c_int]
     L.as_builder_finish_carrier.argtypes = [vp, C.c_uint64, C.POINTER(C.c_int64)]
+    L.as_builder_set_fuse_launches.argtypes = [vp, C.c_int]
+    L.as_builder_launch_is_fused.argtypes = [vp, C.c_uint64]
     L.as_builder_time_sub_matrix.argtypes = [vp, C.c_int64, C.c_uint64, C.POINTER(C.c_float), C.POINTER(C.c_uint64),
                                              C.POINTER(C.c_uint64), C.POINTER(C.c_int)]
     L.as_builder_time_sub_matrix_pass.argtypes = [vp, C.c_int64, C.c_int, C.c_uint64, C.POINTER(C.c_float)]
@@ -76,10 +78,13 @@ def _bind(L):
     _bound = True
 
 
-def device_facts(read_device=None, cu_num=0, lds_bytes=0):
+def device_facts(read_device=None, cu_num=0, lds_bytes=0, reset=False):
     """What the format builders assume about the GPU, as a dict (cu_num, lds_bytes, xcd_num, l2_bytes_per_xcd,
-    from_device).  read_device = a GPU number: ask that GPU first; cu_num / lds_bytes != 0: set them first."""
+    from_device).  read_device = a GPU number: ask that GPU first; cu_num / lds_bytes != 0: set them first;
+    reset: back to the MI355X values first."""
     L = capi.lib()
+    if reset and L.as_device_facts_reset() != 0:
+        raise capi.AlphaSparseError(L.as_last_error().decode())
     L.as_device_facts.argtypes = [capi.u64p, capi.u64p, capi.u64p, capi.u64p, capi.intp]
     L.as_device_facts_set.argtypes = [C.c_uint64, C.c_uint64]
     L.as_device_facts_read.argtypes = [C.c_int]
@@ -392,6 +397,16 @@ class Builder:
     def set_serial_launch(self, serial=True):
         self._chk(self._L.as_builder_set_serial_launch(self._h, int(bool(serial))))
         return self
+
+    def set_fuse_launches(self, on=True):
+        """With a carried finish and equal workgroup sizes: the first kernels of the tile strip and of the product-bin
+        strip behind it as one launch (default on)."""
+        self._chk(self._L.as_builder_set_fuse_launches(self._h, int(bool(on))))
+        return self
+
+    def launch_is_fused(self, sub):
+        """True when the strip behind `sub` runs the trips of its first kernel (a whole SpMV launches nothing for `sub`)."""
+        return bool(self._chk(self._L.as_builder_launch_is_fused(self._h, sub)))
 
     def set_finish_carry(self, on=True):
         """With serial launch: let the first kernel of a product-bin strip do the work of the finish kernel of the

@@ -30,6 +30,13 @@ int as_device_facts_read(int device) {
   AS_API_END(-1)
 }
 
+int as_device_facts_reset(void) {
+  AS_API_BEGIN
+  asx::reset_device_facts();
+  return 0;
+  AS_API_END(-1)
+}
+
 int as_device_facts_set(uint64_t cu_num, uint64_t lds_bytes) {
   AS_API_BEGIN
   AS_CHECK(lds_bytes == 0 || lds_bytes >= 65536, "at least 64 KB of LDS per workgroup");

@@ -325,6 +325,26 @@ int as_builder_set_finish_carry(as_builder *b, int on) {
   AS_API_END(-1)
 }
 
+int as_builder_set_fuse_launches(as_builder *b, int on) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b, "null builder");
+  if (b->b->fuse_launches != (on != 0)) asx::invalidate_module(*b->b);
+  b->b->fuse_launches = on != 0;
+  return 0;
+  AS_API_END(-1)
+}
+
+int as_builder_launch_is_fused(as_builder *b, uint64_t sub) {
+  AS_API_BEGIN
+  AS_CHECK(b && b->b, "null builder");
+  AS_CHECK(sub < b->b->subs.size() && b->b->subs[sub].tpl, "sub-matrix has no template");
+  asx::assign_finish_carriers(*b->b, sub);
+  for (auto &k : b->b->subs)
+    if (k.tpl && k.tpl->fused_trips == b->b->subs[sub].tpl.get()) return 1;
+  return 0;
+  AS_API_END(-1)
+}
+
 int as_builder_finish_carrier(as_builder *b, uint64_t sub, int64_t *carrier) {
   AS_API_BEGIN
   AS_CHECK(b && b->b && carrier, "null argument");

@@ -9,7 +9,7 @@
 
 namespace asx {
 
-static const size_t kMaxKernelArgs = 32;
+static const size_t kMaxKernelArgs = 64;
 
 #define HIPL(call)                                                                      \
   do {                                                                                  \
@@ -233,13 +233,30 @@ int64_t assign_finish_carriers(const Builder &b, uint64_t sub) {
     if (!k.tpl) continue;
     k.tpl->carried = nullptr;
     k.tpl->carried_blocks = 0;
+    k.tpl->fused_trips = nullptr;
     // the strip before leaves its rows in a scratch vector for a finish kernel, and this one starts with a kernel
     // that does not touch y: the two are independent, and the rows of the strip before are this kernel's to move
     if (b.serial_launch && b.carry_finish && before && before->tpl->type == SHARED_MEMORY_TILE_TEMPLATE &&
         before->tpl->finish_tblock_num && before->tpl->scratch_bytes && k.tpl->type == SHARED_MEMORY_PRODUCT_BIN_TEMPLATE) {
-      const uint64_t rows = before->tpl->sc("sub_rows"), threads = std::max<uint64_t>(64, k.tpl->thread_num_in_block);
       k.tpl->carried = before->tpl.get();
+      // With workgroups of the same size the two strips' first kernels become one launch as well: every workgroup
+      // runs a trip of the strip before and then trips of this one, so the tail of the one and the start of the other
+      // overlap CU by CU instead of meeting at a kernel boundary; the carried rows then wait for this strip's SECOND
+      // kernel, which starts when every trip is done.
+      if (b.fuse_launches && before->tpl->thread_num_in_block == k.tpl->thread_num_in_block) k.tpl->fused_trips = before->tpl.get();
+      const uint64_t rows = before->tpl->sc("sub_rows");
+      const uint64_t threads = std::max<uint64_t>(64, k.tpl->fused_trips ? k.tpl->finish_thread_num : k.tpl->thread_num_in_block);
       k.tpl->carried_blocks = std::min<uint64_t>(256, ((rows + threads - 1) / threads + 7) / 8 * 8);
+      if (k.tpl->fused_trips) {
+        // The second kernel's own workgroups are all on the device at once where they fit (two of 1024 threads per
+        // CU): carriers on top of them would be a second round of workgroups, a tail of a few microseconds behind
+        // the first.  As many carriers as still fit the first round, at least eight; each then moves more rows.
+        const uint64_t per_cu = std::max<uint64_t>(1, std::min<uint64_t>(2048 / std::max<uint64_t>(64, k.tpl->finish_thread_num),
+                                                                       device_facts().lds_bytes / std::max<uint64_t>(1, k.tpl->finish_lds_bytes)));
+        const uint64_t room = device_facts().cu_num * per_cu;
+        if (k.tpl->finish_tblock_num <= room && k.tpl->finish_tblock_num + k.tpl->carried_blocks > room)
+          k.tpl->carried_blocks = std::max<uint64_t>(8, (room - k.tpl->finish_tblock_num) / 8 * 8);
+      }
       if (before->tpl->sub == sub) carrier_of_sub = (int64_t)k.tpl->sub;
     }
     before = &k;
@@ -405,55 +422,76 @@ static void launch_kernels(Builder &b, void *stream, const void *x_dev, void *y_
     if (k.tpl->type == EMPTY_TEMPLATE) continue;  // nothing to launch: its rows of y are the clear's
     AS_CHECK(k.uploaded && k.fn, "a template was changed after upload: call upload again");
     // kernel arguments: passed metadata arrays, val, col, x, y, scratch -- a fixed-size list, nothing allocated
-    void *ptrs[kMaxKernelArgs], *args[kMaxKernelArgs];
+    void *ptrs[kMaxKernelArgs], *first_args[kMaxKernelArgs], *finish_args[kMaxKernelArgs];
     size_t n = 0;
-    AS_CHECK(k.meta.size() + 8 <= kMaxKernelArgs, "too many kernel arguments");
-    for (auto &m : k.meta) ptrs[n++] = m.ptr;
-    ptrs[n++] = k.val.ptr;
-    ptrs[n++] = k.col.ptr;
-    ptrs[n++] = (void *)x_dev;
-    ptrs[n++] = y_dev;
-    if (k.tpl->scratch_bytes) ptrs[n++] = scratch_ptr;
-    for (size_t i = 0; i < n; i++) args[i] = &ptrs[i];
-    // A first kernel that carries the finish of the strip before it takes that strip's scratch vector, its places
-    // in y and its number of rows behind its own arguments -- 0 rows when this strip is launched alone.
-    size_t n_first = n;
-    unsigned int carried_rows = 0;
+    auto push_arrays = [&](const SubKernel &from, void *from_scratch) {
+      AS_CHECK(n + from.meta.size() + 8 <= kMaxKernelArgs, "too many kernel arguments");
+      for (auto &m : from.meta) ptrs[n++] = m.ptr;
+      ptrs[n++] = from.val.ptr;
+      ptrs[n++] = from.col.ptr;
+      ptrs[n++] = (void *)x_dev;
+      ptrs[n++] = y_dev;
+      if (from.tpl->scratch_bytes) ptrs[n++] = from_scratch;
+    };
+    push_arrays(k, scratch_ptr);
+    const size_t n_own = n;
+    for (size_t i = 0; i < n_own; i++) first_args[i] = finish_args[i] = &ptrs[i];
+    size_t n_first = n_own, n_finish = n_own;
+    // A kernel that carries the finish of the strip before it takes that strip's scratch vector, its places in y and
+    // its number of rows behind its own arguments -- 0 rows when this strip is launched alone.  With a fused launch
+    // the first kernel takes all arrays of the strip before instead (and a flag: 0 when this strip is launched alone),
+    // and the second kernel carries.
+    unsigned int carried_rows = 0, fused_on = 0;
     if (k.tpl->carried) {
       AS_CHECK(guest && guest->tpl.get() == k.tpl->carried && guest->uploaded, "a template was changed after upload: call upload again");
-      ptrs[n_first] = guest_scratch;
-      args[n_first] = &ptrs[n_first];
-      n_first++;
+      void **carrier_args = k.tpl->fused_trips ? finish_args : first_args;
+      size_t &n_carrier = k.tpl->fused_trips ? n_finish : n_first;
+      ptrs[n] = guest_scratch;
+      carrier_args[n_carrier++] = &ptrs[n++];
       if (carried_place_is_passed(*guest->tpl)) {
         size_t at = 0;
         for (auto &a : guest->tpl->arrays) {
           if (a.name == "y_row_index") break;
           at += a.passed();
         }
-        ptrs[n_first] = guest->meta[at].ptr;
-        args[n_first] = &ptrs[n_first];
-        n_first++;
+        ptrs[n] = guest->meta[at].ptr;
+        carrier_args[n_carrier++] = &ptrs[n++];
       }
       if (b.only_sub < 0) carried_rows = (unsigned int)guest->tpl->sc("sub_rows");
-      args[n_first++] = &carried_rows;
+      carrier_args[n_carrier++] = &carried_rows;
+      if (k.tpl->fused_trips) {
+        const size_t guest_first = n;
+        push_arrays(*guest, guest_scratch);
+        for (size_t i = guest_first; i < n; i++) first_args[n_first++] = &ptrs[i];
+        fused_on = b.only_sub < 0 ? 1u : 0u;
+        first_args[n_first++] = &fused_on;
+      }
     }
-    // ... and the strip before it then launches no finish kernel of its own
-    bool finish_is_carried = false;
+    // ... and the strip before it then launches no finish kernel of its own (with a fused launch: no kernel at all)
+    bool finish_is_carried = false, trips_are_fused = false;
     if (b.only_sub < 0)
       for (size_t j = idx + 1; j < b.subs.size(); j++)
         if (b.subs[j].tpl) {
           finish_is_carried = b.subs[j].tpl->carried == k.tpl.get();
+          trips_are_fused = b.subs[j].tpl->fused_trips == k.tpl.get();
           break;
         }
     void *s = multi ? k.stream : stream;
     if (multi) HIPL(as_hip_stream_wait_event(s, b.start_ev));
-    if (b.only_pass != 2)
-      HIPL(as_hip_launch(k.fn, (unsigned)(k.tpl->tblock_num + k.tpl->carried_blocks), (unsigned)k.tpl->thread_num_in_block,
-                         (unsigned)k.tpl->dynamic_lds_bytes, s, args));
+    if (b.only_pass != 2 && !trips_are_fused) {
+      uint64_t grid = k.tpl->tblock_num, lds = k.tpl->dynamic_lds_bytes;
+      if (k.tpl->fused_trips && fused_on) {
+        grid = std::max(grid, guest->tpl->tblock_num);
+        lds = std::max(lds, guest->tpl->dynamic_lds_bytes);
+      } else if (!k.tpl->fused_trips) {
+        grid += k.tpl->carried_blocks;
+      }
+      HIPL(as_hip_launch(k.fn, (unsigned)grid, (unsigned)k.tpl->thread_num_in_block, (unsigned)lds, s, first_args));
+    }
     if (k.tpl->finish_tblock_num && b.only_pass != 1 && !finish_is_carried) {
       AS_CHECK(k.finish_fn, "a template was changed after upload: call upload again");
-      HIPL(as_hip_launch(k.finish_fn, (unsigned)k.tpl->finish_tblock_num, (unsigned)k.tpl->finish_thread_num,
-                         (unsigned)k.tpl->finish_lds_bytes, s, args));
+      HIPL(as_hip_launch(k.finish_fn, (unsigned)(k.tpl->finish_tblock_num + (k.tpl->fused_trips ? k.tpl->carried_blocks : 0)),
+                         (unsigned)k.tpl->finish_thread_num, (unsigned)k.tpl->finish_lds_bytes, s, finish_args));
     }
     if (multi) {
       HIPL(as_hip_event_record(k.done, s));

@@ -47,6 +47,9 @@ struct Builder {
   // product-bin template; the first workgroups of that template's first kernel do its work instead (see
   // assign_finish_carriers).  false: every template launches its own kernels.
   bool carry_finish = true;
+  // With a carried finish and workgroups of the same size in both strips: the first kernels of the two strips are
+  // one launch (Template::fused_trips).  false: two launches.
+  bool fuse_launches = true;
   // >= 0: launches and timing cover the kernels of this sub-matrix only (per-kernel measurement)
   int64_t only_sub = -1;
   int only_pass = 0;  // with only_sub: 1 = the first kernel alone, 2 = the finish kernel alone, 0 = both

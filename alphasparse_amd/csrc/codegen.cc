@@ -97,16 +97,29 @@ template <int LANES, typename T> __device__ __forceinline__ T as_group_sum_shfl(
 )SRC";
 }
 
-std::string kernel_signature(const Template &t) {
+std::string kernel_signature(const Template &t) { return kernel_signature(t, std::string()); }
+
+std::string kernel_signature(const Template &t, const std::string &p) {
   std::string s;
   for (auto &a : t.arrays)
-    if (a.passed()) s += std::string("const ") + dtype_c_name(a.a.dt) + " *__restrict__ " + a.name + ", ";
+    if (a.passed()) s += std::string("const ") + dtype_c_name(a.a.dt) + " *__restrict__ " + p + a.name + ", ";
   std::string vt = value_type_name(t);
-  s += "const " + vt + " *__restrict__ val_arr, const " + std::string(dtype_c_name(t.col_index_arr.dt)) +
-       " *__restrict__ col_index_arr, const " + vt + " *__restrict__ device_x_arr, " + vt + " *__restrict__ device_y_arr";
-  if (t.scratch_bytes) s += ", unsigned int *__restrict__ scratch_arr";
+  s += "const " + vt + " *__restrict__ " + p + "val_arr, const " + std::string(dtype_c_name(t.col_index_arr.dt)) +
+       " *__restrict__ " + p + "col_index_arr, const " + vt + " *__restrict__ " + p + "device_x_arr, " + vt + " *__restrict__ " + p + "device_y_arr";
+  if (t.scratch_bytes) s += ", unsigned int *__restrict__ " + p + "scratch_arr";
   return s;
 }
+
+std::string kernel_arguments(const Template &t, const std::string &p) {
+  std::string s;
+  for (auto &a : t.arrays)
+    if (a.passed()) s += p + a.name + ", ";
+  s += p + "val_arr, " + p + "col_index_arr, " + p + "device_x_arr, " + p + "device_y_arr";
+  if (t.scratch_bytes) s += ", " + p + "scratch_arr";
+  return s;
+}
+
+std::string kernel_trips_function_name(const Template &t) { return "spmv_" + std::to_string(t.sub) + "_trips"; }
 
 bool carried_place_is_passed(const Template &guest) { return guest.arr("y_row_index").passed(); }
 

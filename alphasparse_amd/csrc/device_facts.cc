@@ -38,4 +38,10 @@ void set_device_facts(uint64_t cu_num, uint64_t lds_bytes) {
   g_facts.from_device = true;
 }
 
+
+void reset_device_facts() {
+  std::lock_guard<std::mutex> lock(g_facts_mutex);
+  g_facts = DeviceFacts();
+}
+
 }  // namespace asx

@@ -26,5 +26,7 @@ uint64_t x_slice_bytes();
 void read_device_facts(int device);
 // For callers that build formats for a GPU they cannot ask (another partition mode, tests): 0 keeps a value.
 void set_device_facts(uint64_t cu_num, uint64_t lds_bytes);
+// back to the MI355X values, to be read from a GPU again at the next upload or search
+void reset_device_facts();
 
 }  // namespace asx

@@ -351,9 +351,23 @@ std::vector<TemplateNode> launch_candidates(const Template &t) {
 // find_best_template_node_of_specific_sub_matrix_from_template_set (default_auto_tuner.cc:44):
 // best (template, launch parameters) for an already built format of one sub-matrix
 bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<TemplateType> &types, SearchStrategy *local,
-                        TemplateNode &best, float &best_gflops, float &best_ms, const MatrixInfo *info = nullptr) {
+                        TemplateNode &best, float &best_gflops, float &best_ms, const MatrixInfo *info = nullptr,
+                        uint64_t *best_bytes = nullptr) {
   best_gflops = 0;
   best_ms = 0;
+  // useful bytes the best kernel so far moves per launch: its format arrays (scratch written and read included), x
+  // once and the strip's rows of y once -- noted whenever `best` changes
+  float noted_ms = -1;
+  auto note_bytes = [&](const Builder &b) {
+    if (!best_bytes || best_ms == noted_ms || !b.subs[sub].tpl) return;
+    const uint64_t vs = (uint64_t)dtype_size(m.val_dtype);
+    const uint64_t strip_rows = m.items[sub].max_row - m.items[sub].min_row + 1;
+    const uint64_t format = template_format_bytes(*b.subs[sub].tpl) + m.cols * vs + strip_rows * vs;
+    // ... but no more than a CSR of the strip with 32-bit columns would move: padding is not useful work
+    const uint64_t csr = b.subs[sub].tpl->origin_nnz * (vs + 4) + (strip_rows + 1) * 4 + (m.cols + strip_rows) * vs;
+    *best_bytes = std::min(format, csr);
+    noted_ms = best_ms;
+  };
   execute_default_div_to_complete_each_level_blocking(m, sub);
   const CompressedBlock &cb = *m.items[sub].cb;
   double rate = (double)cb.padding_val->size() / (double)cb.read_index[0]->length;
@@ -417,7 +431,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
               " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
               (n.col_relative == 3 ? " column runs," : "") + " row ownership, row blocks of " + std::to_string(n.row_block) +
               " -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us" + c.stamp());
-        if (gf > best_gflops * (best_gflops > 0 && best.type == type ? 1.01f : 1.0f)) { best_gflops = gf; best_ms = ms; best = n; }
+        if (gf > best_gflops * (best_gflops > 0 && best.type == type ? 1.01f : 1.0f)) { best_gflops = gf; best_ms = ms; best = n; note_bytes(*b); }
         bool go = local ? continue_search(*local, gf) : true;
         if (!go || !continue_search(c.global)) return best_gflops > 0;
       }
@@ -456,12 +470,15 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
       // another launch setting of the template that leads must lead by more than the noise of two timings (1 %):
       // the same matrix then gets the same graph from one search to the next
       const bool same_template = best_gflops > 0 && best.type == type;
-      if (gf > best_gflops * (same_template ? 1.01f : 1.0f)) { best_gflops = gf; best_ms = ms; best = n; }
+      if (gf > best_gflops * (same_template ? 1.01f : 1.0f)) { best_gflops = gf; best_ms = ms; best = n; note_bytes(*b); }
       bool go = local ? continue_search(*local, gf) : true;
-      if (gf > c.global.best_glops) {
-        // time-to-best bookkeeping uses the global clock
-      }
       if (!go || !continue_search(c.global)) return best_gflops > 0;
+      // launch settings of one format differ by tens of percent, not by factors: a format whose first setting alone
+      // takes more than twice the best whole SpMV so far is not swept
+      if (c.best_whole_ms > 0 && ms > 2.0f * c.best_whole_ms) {
+        c.log("  first launch setting alone takes more than 2 x the best whole SpMV so far, other settings skipped");
+        break;
+      }
     }
     // the best launch of the ELL template once more with 16-bit relative columns and then with the columns
     // computed from the slots' diagonals, where the matrix allows them
@@ -483,7 +500,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
                 " threads " + std::to_string(n.thread_num_in_block) + " vec " + std::to_string(n.vec_width) +
                 (form == 1 ? " relative columns -> " : " diagonal columns -> ") + std::to_string(gf) + " GFLOP/s, " +
                 std::to_string(ms * 1e3f) + " us");
-          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; note_bytes(*b); }
         } catch (const std::exception &e) {
           c.res.failed_candidates++;
           c.log(std::string("  candidate failed: ") + e.what());
@@ -507,7 +524,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
           c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
                 " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
                 " column runs -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
-          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; note_bytes(*b); }
         }
       } catch (const std::exception &e) {
         c.res.failed_candidates++;
@@ -535,7 +552,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
           c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
                 " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
                 " row ownership -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
-          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+          if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; note_bytes(*b); }
           // and, where the rows come in blocks that hold the same columns, with a block of rows as one piece
           const uint64_t height = best.own_rows == 1 ? tile_row_block_guess(m, sub) : 1;
           if (height > 1 && set_row_blocks(*b, sub, height)) {
@@ -552,7 +569,7 @@ bool find_best_template(Ctx &c, Matrix &m, uint64_t sub, const std::vector<Templ
             c.log(std::string("  template sub_matrix_id:") + std::to_string(sub) + " " + convert_template_type_to_string(type) +
                   " threads " + std::to_string(n.thread_num_in_block) + " blocks " + std::to_string(n.tblock_num) +
                   " row blocks of " + std::to_string(height) + " -> " + std::to_string(gf) + " GFLOP/s, " + std::to_string(ms * 1e3f) + " us");
-            if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; }
+            if (gf > best_gflops) { best_gflops = gf; best_ms = ms; best = n; note_bytes(*b); }
           }
         }
       } catch (const std::exception &e) {
@@ -835,6 +852,8 @@ std::vector<Skeleton> skeletons_for(const MatrixInfo &info, bool globally_sorted
 }
 
 constexpr float kFamilyCutoff = 5.0f;
+constexpr double kStreamingFrac = 0.62;
+constexpr double kHbmPeakBytesPerSecond = 8e12;   // MI355X, HBM3E
 constexpr float kWholeCutoff = 2.0f;
 
 // find_best_path_of_compressed_sub_matrix (whilte_list_path_impl.cc:3411)
@@ -872,20 +891,32 @@ bool find_best_path_of_compressed_sub_matrix(Ctx &c, const Matrix &base, uint64_
       }
       TemplateNode tn;
       float gf = 0, ms = 0;
+      uint64_t fmt_bytes = 0;
       bool ok = false;
       try {
-        ok = find_best_template(c, *m, sub, sk.templates, &local, tn, gf, ms, &info);
+        ok = find_best_template(c, *m, sub, sk.templates, &local, tn, gf, ms, &info, &fmt_bytes);
       } catch (const std::exception &ex) {
         c.res.failed_candidates++;
         c.log(std::string("  candidate failed: ") + ex.what());
       }
       if (ok && gf > best.gflops) {
         best.gflops = gf; best.time_ms = ms; best.tpl = tn;
+        best.format_bytes = fmt_bytes;
         best.found_at_s = c.now_s();
         best.nodes = nodes;
         for (auto &n : best.nodes) n.node.reset_param();  // the graph keeps knobs, not expanded parameters
       }
       if (!continue_search(local) || !continue_search(c.global)) return best.gflops > 0;
+      // A kernel that moves its format (+ x and the strip's rows of y; at most what a CSR of the strip would move) at
+      // more than kStreamingFrac of the HBM peak is close to what a plain copy reaches on this device (0.75-0.78):
+      // the skeletons and settings not tried yet could only win by a format of far fewer bytes, and the compact
+      // formats are the ones in front.
+      if (ok && best.time_ms > 0 && best.format_bytes > 0 &&
+          (double)best.format_bytes / ((double)best.time_ms * 1e-3) > kStreamingFrac * kHbmPeakBytesPerSecond) {
+        c.log("  the strip's kernel moves its format at more than " + std::to_string(kStreamingFrac) +
+              " of the HBM peak: the remaining settings and skeletons are not tried" + c.stamp());
+        return true;
+      }
       // a family whose first setting runs at under a fifth of the strip's best is not swept further: its
       // settings differ among themselves by far less than that
       if (first_knob && ok && gf * kFamilyCutoff < best.gflops) {
@@ -962,17 +993,68 @@ bool search_dense_strategy(Ctx &c, const CooInput &in, std::vector<StrategyNode>
     BuiltGraph bg = build_from_graph(in, out, c.opt.wave);
     load_and_upload(*bg.builder, c.opt.device);
     if (as_hip_h2d(bg.builder->x.ptr, c.probe_x.data(), bg.builder->x.bytes) != 0) throw Error(as_hip_last_error());
-    verify_candidate(c, *bg.builder, *bg.matrix, -1);
-    time_builder(c, *bg.builder, out.time_ms, out.gflops);
+    // Strip kernels that each take whole CUs (the LDS-tile templates: one or two workgroups fill a CU's LDS) only
+    // get in each other's way on concurrent streams -- measured on every such graph so far (C3: 737 against 1042
+    // GFLOP/s, C5: 540 against 632) -- so that way of launching is measured only where a strip has a kernel of
+    // another kind.
+    bool whole_cu_kernels = true;
+    for (auto &sg : out.subs)
+      whole_cu_kernels = whole_cu_kernels && (sg.tpl.type == SHARED_MEMORY_TILE_TEMPLATE || sg.tpl.type == SHARED_MEMORY_PRODUCT_BIN_TEMPLATE);
+    if (!whole_cu_kernels) {
+      verify_candidate(c, *bg.builder, *bg.matrix, -1);
+      time_builder(c, *bg.builder, out.time_ms, out.gflops);
+    }
     // kernels that each fill the machine can be faster one after the other than on concurrent streams
     float ms = 0, gf = 0;
     bg.builder->serial_launch = true;
     invalidate_module(*bg.builder);  // one after the other a finish kernel may be carried by the next strip's kernel
     verify_candidate(c, *bg.builder, *bg.matrix, -1);
     time_builder(c, *bg.builder, ms, gf);
-    c.log("combined graph: " + std::to_string(out.gflops) + " GFLOP/s on concurrent streams, " + std::to_string(gf) + " one after the other" + c.stamp());
+    c.log("combined graph: " + (whole_cu_kernels ? std::string("not measured") : std::to_string(out.gflops) + " GFLOP/s") +
+          " on concurrent streams, " + std::to_string(gf) + " GFLOP/s one after the other" + c.stamp());
     if (gf > out.gflops) { out.gflops = gf; out.time_ms = ms; out.serial_launch = true; }
     out.found_at_s = c.now_s();
+    // A tile strip in front of a product-bin strip with workgroups of another size: with the same size in both, their
+    // first kernels are one launch (Template::fused_trips).  Both common sizes are measured; the strips were tuned
+    // one by one, the launch boundary between them is the whole graph's business.
+    if (out.serial_launch)
+      for (size_t i = 0; i + 1 < out.subs.size(); i++) {
+        TemplateNode &tile = out.subs[i].tpl, &bin = out.subs[i + 1].tpl;
+        if (tile.type != SHARED_MEMORY_TILE_TEMPLATE || bin.type != SHARED_MEMORY_PRODUCT_BIN_TEMPLATE ||
+            tile.thread_num_in_block == bin.thread_num_in_block || assign_finish_carriers(*bg.builder, i) != (int64_t)(i + 1))
+          continue;
+        const long sizes[2] = {tile.thread_num_in_block, bin.thread_num_in_block};
+        for (long threads : sizes) {
+          TemplateNode t2 = tile, b2 = bin;
+          t2.thread_num_in_block = b2.thread_num_in_block = threads;
+          t2.tblock_num = b2.tblock_num = 0;
+          try {
+            set_launch(*bg.builder->subs[i].tpl, t2);
+            set_launch(*bg.builder->subs[i + 1].tpl, b2);
+            invalidate_module(*bg.builder);
+            verify_candidate(c, *bg.builder, *bg.matrix, -1);
+            time_builder(c, *bg.builder, ms, gf);
+          } catch (const std::exception &e) {
+            c.res.failed_candidates++;
+            c.log(std::string("  candidate failed: ") + e.what());
+            continue;
+          }
+          c.res.candidates++;
+          c.log("combined graph, both strips with " + std::to_string(threads) + " threads (one launch for their first kernels): " +
+                std::to_string(gf) + " GFLOP/s" + c.stamp());
+          if (gf > out.gflops * 1.005f) {
+            out.gflops = gf; out.time_ms = ms;
+            t2.tblock_num = (long)bg.builder->subs[i].tpl->tblock_num;
+            b2.tblock_num = (long)bg.builder->subs[i + 1].tpl->tblock_num;
+            tile = t2; bin = b2;
+            out.found_at_s = c.now_s();
+          }
+        }
+        // leave the builder with the launch settings that won
+        set_launch(*bg.builder->subs[i].tpl, tile);
+        set_launch(*bg.builder->subs[i + 1].tpl, bin);
+        invalidate_module(*bg.builder);
+      }
   } catch (const std::exception &e) {
     c.log(std::string("combined graph failed: ") + e.what());
     return false;
@@ -1143,7 +1225,7 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
       // than an XCD's L2 cache; then the upstream grid 512/128/32 x 4/8/16 with bands up to 2048.
       std::vector<std::array<long, 3>> bands;
       if (in.col_index_max + 1 > kL2BytesPerXcd / (in.val_dtype == DOUBLE ? 8 : 4))
-        for (long low : {64, 16, 256}) bands.push_back({low, low, 2});
+        for (long low : {48, 16, 256}) bands.push_back({low, low, 2});
       for (long low : {512, 128, 32})
         for (long rate : {4, 8, 16}) bands.push_back({low, 2048, rate});
       std::vector<std::vector<uint64_t>> seen;
@@ -1160,7 +1242,8 @@ SearchResult find_best_graph_of_white_list_strategy(const CooInput &in, const Se
         c.global = init_search_strategy(opt.struggle_step_num, T - now_s());
         BestGraph g;
         double budget = (T - now_s()) / 2;
-        if (search_dense_strategy(c, in, {input, sort, div, compress}, budget, g) && g.gflops > best3.gflops) {
+        // another row division must lead by more than the noise of two timings (1 %), as launch settings must
+        if (search_dense_strategy(c, in, {input, sort, div, compress}, budget, g) && g.gflops > best3.gflops * 1.01f) {
           best3 = g;
           struggle = 0;
         } else if (best3.gflops > 0 && ++struggle >= 3) {

@@ -72,6 +72,7 @@ struct SubGraph {
   std::vector<StrategyNode> nodes;
   TemplateNode tpl;
   float gflops = 0, time_ms = 0;
+  uint64_t format_bytes = 0;  // bytes the kernel moves per launch: format arrays, x once, the strip's rows of y once
   double found_at_s = 0;  // seconds into the search at which this candidate was measured
 };
 // dense_view_matrix_and_compressed_sub_block_exe_graph_and_template_t

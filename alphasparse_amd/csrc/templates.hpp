@@ -93,6 +93,12 @@ struct Template {
   // Not owned; nullptr = none.
   const Template *carried = nullptr;
   uint64_t carried_blocks = 0;
+  // Fused launch (set by the builder together with `carried`, see assign_finish_carriers): this template's first
+  // kernel runs the trips of the first kernel of `fused_trips` -- the template of the row strip in front of it, the
+  // same as `carried` -- ahead of its own, workgroup by workgroup, so that strip launches nothing of its own; the
+  // carried finish then moves to THIS template's finish kernel (everything of the strip in front must be done
+  // before its row sums are read).  Not owned; nullptr = none.
+  const Template *fused_trips = nullptr;
   // LDS the kernel asks for at launch (beyond its static __shared__ arrays)
   uint64_t dynamic_lds_bytes = 0;
   // Device scratch of the kernels (last argument `scratch_arr`): allocated and cleared once at upload; what
@@ -216,6 +222,13 @@ std::string kernel_module_preamble();
 // "const <type>* __restrict__ <name>, " for every passed metadata array, then
 // val/col/x/y.
 std::string kernel_signature(const Template &t);
+// the same with every parameter name behind `prefix` (a kernel that takes the arrays of two templates), and the
+// matching argument list "prefix + name, ..." for a call
+std::string kernel_signature(const Template &t, const std::string &prefix);
+std::string kernel_arguments(const Template &t, const std::string &prefix);
+// Name of the device function that holds the body of a template's first kernel, for templates whose trips another
+// template's kernel can run (the tile template): (kernel_signature, unsigned as_block, unsigned as_grid).
+std::string kernel_trips_function_name(const Template &t);
 // A kernel that can carry another template's finish (Template::carried) appends carried_finish_signature to its
 // parameters and opens its body with carried_finish_prologue: the code of the carrying workgroups, then the
 // definitions of as_block / as_grid, the number of this workgroup among the kernel's own and how many those are.

@@ -355,9 +355,27 @@ std::string kernel_source(const Template &t) {
   const bool wide_copy = t.kernal_first_col_index % 4 == 0;
   std::string s;
   // ---- first pass: products -------------------------------------------------------------------
+  // Fused launch: the workgroups first run the trips of the strip in front of this one (its arrays behind this
+  // kernel's own, `fused_on` = 0 when this strip is launched alone), then their own; the carried finish is then the
+  // second kernel's.  Otherwise the first workgroups of this kernel carry the finish (carried_finish_prologue).
+  const Template *fused = t.fused_trips;
+  AS_CHECK(!fused || (fused == t.carried && fused->thread_num_in_block == t.thread_num_in_block),
+           "a fused launch needs the same workgroup size in both strips");
   s += "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(t.thread_num_in_block) + ") spmv_" + id + "(" +
-       kernel_signature(t) + carried_finish_signature(t) + ")\n{\n";
-  s += carried_finish_prologue(t, t.thread_num_in_block);
+       kernel_signature(t) + (fused ? ", " + kernel_signature(*fused, "fused_") + ", unsigned int fused_on" : carried_finish_signature(t)) + ")\n{\n";
+  if (fused) {
+    // The launch has as many workgroups as the longer of the two lists of trips.  Each list is dealt out among its
+    // own first workgroups only (workgroup i runs on XCD i % 8, and the XCD-contiguous numbering of the trips
+    // assumes that the workgroups that share them are numbered 0, 1, 2, ...): numbered over the whole launch, the
+    // trips of the shorter list would all land on the first XCDs.
+    const std::string G0 = std::to_string(fused->tblock_num) + "u";
+    s += "  if (fused_on && blockIdx.x < " + G0 + ")\n  {\n    " + kernel_trips_function_name(*fused) + "(" + kernel_arguments(*fused, "fused_") + ", blockIdx.x, " + G0 + ");\n";
+    s += "    __syncthreads();\n  }\n";   // the LDS is this kernel's from here on
+    s += "  const unsigned int as_block = blockIdx.x, as_grid = min(gridDim.x, " + std::to_string(t.tblock_num) + "u);\n";
+    s += "  if (as_block >= as_grid) return;\n";
+  } else {
+    s += carried_finish_prologue(t, t.thread_num_in_block);
+  }
   const std::string Cs = std::to_string(16 / dtype_size(t.val_dtype));
   s += "  typedef " + vt + " val16_t __attribute__((ext_vector_type(" + Cs + ")));\n";  // 16 bytes of values
   s += "  extern __shared__ __attribute__((aligned(16))) unsigned char as_dynamic_lds[];\n";
@@ -436,7 +454,10 @@ std::string kernel_source(const Template &t) {
   // elements: lane j of every wavefront holds first[j], read with v_readlane -- no LDS round trip between two
   // elements of a row.  Wider rows: a table in LDS.
   const bool table_in_register = t.sc("max_width") <= 63;
-  s += "extern \"C\" __global__ void __launch_bounds__(" + FB + ") spmv_" + id + "_finish(" + kernel_signature(t) + ")\n{\n";
+  s += "extern \"C\" __global__ void __launch_bounds__(" + FB + ") spmv_" + id + "_finish(" + kernel_signature(t) +
+       (fused ? carried_finish_signature(t) : std::string()) + ")\n{\n";
+  if (fused) s += carried_finish_prologue(t, FBn);
+  else s += "  const unsigned int as_block = blockIdx.x, as_grid = gridDim.x;\n";
   s += "  extern __shared__ __attribute__((aligned(16))) unsigned char as_dynamic_lds[];\n";
   if (!table_in_register) s += "  __shared__ unsigned int first_slot[" + std::to_string(t.sc("max_width") + 1) + "];\n";
   s += "  " + vt + " *slots = (" + vt + " *)as_dynamic_lds;\n";
@@ -444,7 +465,7 @@ std::string kernel_source(const Template &t) {
   s += "  const unsigned int lane = threadIdx.x & 63u, wave_in_block = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);\n";
   s += "  const unsigned int stride = (" + FB + "u >> 6) * 256u;\n";
   // neighbouring bands write neighbouring rows of y: they run on the same XCD, behind the same L2
-  s += "  for (unsigned int grp = as_xcd_block_index(); grp < " + std::to_string(nband) + "u; grp += gridDim.x)\n  {\n";
+  s += "  for (unsigned int grp = as_xcd_block_index(as_block, as_grid); grp < " + std::to_string(nband) + "u; grp += as_grid)\n  {\n";
   s += "    unsigned int next_grp = grp + 1u, unit_begin, unit_end, count_begin, count_end, y_begin;\n";
   s += "    " + code_of_meta_read(t, "band_first_unit", "unit_begin", "grp");
   s += "    " + code_of_meta_read(t, "band_first_unit", "unit_end", "next_grp");

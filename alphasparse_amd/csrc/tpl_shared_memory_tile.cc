@@ -596,8 +596,12 @@ std::string kernel_source(const Template &t) {
   const bool wide_copy = t.kernal_first_col_index % 4 == 0;
   const std::string target = t.scratch_bytes ? "(" + vt + " *)scratch_arr" : "device_y_arr";
   std::string s;
-  s += "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(t.thread_num_in_block) + ") spmv_" + id + "(" +
-       kernel_signature(t) + ")\n{\n";
+  // The body is a device function of its own: the kernel spmv_<id> runs it for its own workgroups, and the first
+  // kernel of the strip behind this one can run it ahead of its own trips (Template::fused_trips).  as_block /
+  // as_grid: the number of the workgroup among those that run the trips, and how many they are.
+  // (C linkage like the kernels: the declaration of the dynamic LDS array inside it must agree with theirs)
+  s += "extern \"C\" __device__ __forceinline__ void " + kernel_trips_function_name(t) + "(" + kernel_signature(t) +
+       ", const unsigned int as_block, const unsigned int as_grid)\n{\n";
   // row blocks: a lane's loads of values cover its eight elements in each of the block's rows
   const unsigned RB = t.scalar.count("row_block") ? (unsigned)t.sc("row_block") : 1u;
   const unsigned chunk = 16 / (unsigned)dtype_size(t.val_dtype), chunks = (unsigned)kLaneElems / chunk;
@@ -617,7 +621,7 @@ std::string kernel_source(const Template &t) {
   s += "  const unsigned int lane = threadIdx.x & 63u, wave_in_block = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);\n";
   s += "  const unsigned int stride = (" + B + " >> 6) * " + Us + ";\n";
   s += "  const " + vt + " *x_sub = device_x_arr + " + std::to_string(t.kernal_first_col_index) + "u;\n";
-  s += "  for (unsigned int grp = as_xcd_block_index(); grp < " + std::to_string(G) + "u; grp += gridDim.x)\n  {\n";
+  s += "  for (unsigned int grp = as_xcd_block_index(as_block, as_grid); grp < " + std::to_string(G) + "u; grp += as_grid)\n  {\n";
   s += "    unsigned int next_grp = grp + 1u, run_begin, run_end;\n";
   s += "    " + code_of_meta_read(t, "group_first_run", "run_begin", "grp");
   s += "    " + code_of_meta_read(t, "group_first_run", "run_end", "next_grp");
@@ -798,6 +802,8 @@ std::string kernel_source(const Template &t) {
     s += "          if (as_is_segment_tail(cell)) " + emit(kLaneElems - 1) + "\n";
   }
   s += "        }\n      }\n    }\n  }\n}\n";
+  s += "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(t.thread_num_in_block) + ") spmv_" + id + "(" +
+       kernel_signature(t) + ")\n{\n  " + kernel_trips_function_name(t) + "(" + kernel_arguments(t, "") + ", blockIdx.x, gridDim.x);\n}\n";
   if (t.finish_tblock_num) {
     s += "extern \"C\" __global__ void __launch_bounds__(256) spmv_" + id + "_finish(" + kernel_signature(t) + ")\n{\n";
     s += "  " + vt + " *row_sum = (" + vt + " *)scratch_arr;\n";

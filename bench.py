@@ -45,12 +45,12 @@ WORKLOADS = {
     "C2": ("C2: 5-point Laplacian, 2048x2048 grid, 4194304 rows, fp32", "laplacian_5pt", {"grid": 2048}, 45.0, 30.0,
            "S5,256,1,dia", 12.0),
     "C3": ("C3: power-law row lengths (Zipf 1.8, mean 16, max 200000), 2000000 rows, uniform columns, fp32", "power_law",
-           {}, 90.0, 60.0, "sort+div64|T1@1024|T2:slice=8192,group=65536@512", 30.0),
+           {}, 90.0, 60.0, "sort+div48|T1@1024|T2:slice=16384,group=4096@1024", 30.0),
     "C4": ("C4: FEM-like dense 3x3 blocks, 27 block columns per block row in a +-2000 band, 1000002 rows, fp64",
            "fem_blocks", {}, 45.0, 25.0, "|T1:slice=16384,group=4092@1024,runs,own,blk3", 35.0),
     "C5": ("C5: 8000000 rows of 1-3 elements + 800 rows of 50000-1000000 elements, uniform columns, fp64",
            "extreme_irregular", {"target_nnz": 60_000_000}, 150.0, 75.0,
-           "sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=65536@256", 45.0),
+           "sort+div16|T1:slice=16384,group=4096@1024|T2:slice=16384,group=4096@1024", 45.0),
 }
 # the rocprofv3 summary that covers each configuration's kernels
 PROFILE_OF = {"C2": "profiles/spmv_ell_c2_laplacian_hbm_traffic.txt", "C3": "profiles/spmv_tile_product_bin_c3_power_law.txt",

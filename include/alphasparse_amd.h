@@ -317,6 +317,16 @@ int as_builder_set_serial_launch(as_builder *b, int serial);
  * current templates and settings, or -1.  No counterpart in the reference. */
 int as_builder_set_finish_carry(as_builder *b, int on);
 int as_builder_finish_carrier(as_builder *b, uint64_t sub, int64_t *carrier);
+/* With a carried finish and the same workgroup size in both strips (default on): the first kernels of the two
+ * strips are ONE launch -- every workgroup runs a trip of the tile strip and then trips of the product-bin strip, so
+ * the end of the one and the start of the other overlap CU by CU instead of meeting at a kernel boundary -- and the
+ * tile strip's rows are moved to y by the first workgroups of the product-bin strip's second kernel.  An SpMV of
+ * such a graph is two launches.  0: every strip launches its first kernel itself.  No counterpart in the
+ * reference, whose generated program launches one kernel per sub-matrix (code_builder.cc:1517-1549). */
+int as_builder_set_fuse_launches(as_builder *b, int on);
+/* 1 when the first kernel of `sub` is run by the first kernel of the strip behind it (so `sub` launches nothing of
+ * its own in a whole SpMV), 0 when not, <0 on error */
+int as_builder_launch_is_fused(as_builder *b, uint64_t sub);
 /* `reps` back-to-back launches of the kernels of one sub-matrix only, timed with events on the launch stream;
  * also returns what that kernel's roofline figure is computed from: the bytes of its format arrays (padded
  * col + val + passed metadata), the rows of its strip and whether it accumulates y atomically.  No
@@ -339,6 +349,8 @@ int as_device_facts(uint64_t *cu_num, uint64_t *lds_bytes, uint64_t *xcd_num, ui
 int as_device_facts_read(int device);
 /* formats for a GPU that cannot be asked (another partition mode; tests): 0 keeps a value */
 int as_device_facts_set(uint64_t cu_num, uint64_t lds_bytes);
+/* back to the MI355X values; the next upload or search asks its GPU again */
+int as_device_facts_reset(void);
 /* fill the builder's own x (used by the timing calls) */
 int as_builder_set_x(as_builder *b, const void *x_host);
 /* `reps` launches timed with events; gflops = 2 * origin_nnz * reps / time (code_builder.cc:1557).

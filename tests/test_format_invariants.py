@@ -545,6 +545,39 @@ def test_tile_template_in_column_run_form(vdt, chunk, sort):
     assert not b.set_column_runs(0)
 
 
+def test_formats_are_sized_for_the_device_they_are_told_about():
+    """The tile and product-bin templates cut their element streams into one trip per workgroup the device holds:
+    built for 128 compute units they have half the trips they have for 256, and a slice of x that needs more LDS
+    than the device gives a workgroup is turned down.  The facts default to an MI355X and are read from the GPU at
+    the first upload or search (here they are set by hand and put back)."""
+    from alphasparse_amd import skeletons as SK
+    rows, cols, r, c, v, x = S.power_law(200000, max_len=3000, mean_len=40.0, seed=4)
+    trips = {}
+    try:
+        for cus in (256, 128):
+            A.device_facts(cu_num=cus)
+            for skel in ("T1", "T2"):
+                m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.FLOAT, wave=64)
+                m.execute_strategy(K.COMPRESS_NONE)
+                b = A.Builder(m)
+                b.set_template(0, SK.apply_skeleton(m, 0, skel, slice=16384, group=4096, b=8192)[0])
+                trips[cus, skel] = b.describe(0)["group_num"]
+        assert A.device_facts() == {"cu_num": 128, "lds_bytes": 163840, "xcd_num": 8, "l2_bytes_per_xcd": 4 << 20, "from_device": True}
+        for skel in ("T1", "T2"):
+            assert trips[256, skel] > 200 and abs(trips[128, skel] * 2 - trips[256, skel]) <= 0.1 * trips[256, skel], trips
+        # 64 KB of LDS per workgroup: a 128 KB slice of x does not fit any more
+        A.device_facts(lds_bytes=65536)
+        m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.FLOAT, wave=64)
+        m.execute_strategy(K.COMPRESS_NONE)
+        tp = SK.apply_skeleton(m, 0, "T1", slice=32768, group=4096, b=8192)[0]
+        assert not A.template_is_supported(m, 0, tp)
+        with pytest.raises(K.AlphaSparseError):
+            A.device_facts(lds_bytes=1000)
+    finally:
+        assert A.device_facts(reset=True) == {"cu_num": 256, "lds_bytes": 163840, "xcd_num": 8, "l2_bytes_per_xcd": 4 << 20,
+                                              "from_device": False}
+
+
 def _matrix_with_a_strip_of_zeros():
     """200 rows of 8 elements with values, then 100 rows of one explicit zero; sorted and cut at row length 2."""
     rng = np.random.default_rng(2)

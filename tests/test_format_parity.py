@@ -177,6 +177,14 @@ def test_format_matches_upstream_live(skel, seed, sort):
     assert p.returncode == 0, "return code %d\n" % p.returncode + p.stdout[-3000:] + p.stderr[-2000:]
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("skel", sorted(RANDOM_SEQS))
+def test_format_matches_upstream_live_on_the_gpu_box(skel):
+    """The same comparison in the suite of the GPU box, where the upstream library travels as a built file:
+    one seed per operator sequence, sorted input."""
+    test_format_matches_upstream_live(skel, 0, True)
+
+
 @pytest.mark.parametrize("skel", ["S1", "S2", "S3", "S6", "S7", "B1", "B2"])
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_block_sort_matches_upstream_live(skel, seed):

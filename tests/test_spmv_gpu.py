@@ -572,7 +572,7 @@ def test_full_laplacian_closed_form_and_linearity(laplacian_full):
 
 # ---- full-size configurations 3, 4 and 5 through the graphs the search returns for them -----------------------
 def _full_c3():
-    return S.power_law(), K.FLOAT, (64, "T1", {}, 1024, False), ("T2", {"slice": 8192, "group": 65536}, 512)
+    return S.power_law(), K.FLOAT, (48, "T1", {}, 1024, False), ("T2", {"slice": 16384, "group": 4096}, 1024)
 
 
 def _full_c4():
@@ -581,7 +581,7 @@ def _full_c4():
 
 def _full_c5():
     return (S.extreme_irregular(target_nnz=60_000_000), K.DOUBLE, (16, "T1", {"slice": 16384, "group": 4096}, 1024, False),
-            ("T2", {"slice": 16384, "group": 65536}, 256))
+            ("T2", {"slice": 16384, "group": 4096}, 1024))
 
 
 @pytest.mark.parametrize("make", [_full_c3, _full_c4, _full_c5], ids=["C3", "C4", "C5"])
@@ -667,8 +667,17 @@ def test_finish_of_a_tile_strip_carried_by_the_next_strips_kernel(gpu, vdt):
         b.compile().upload(gpu)
         src = b.kernel_source()
         assert "carried_sum" in src and "spmv_0_finish" in src and not b.clears_y()
+        # workgroups of the same size in both strips (the tile strip has 1024 threads): one launch for both first kernels
+        assert b.launch_is_fused(0) == (threads == 1024) and ("fused_on" in src) == (threads == 1024)
         print("case: carried finish, %d threads" % threads, flush=True)
         assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, y = NaN before the call")
+        if threads == 1024:
+            b.set_fuse_launches(False)
+            b.compile().upload(gpu)
+            assert not b.launch_is_fused(0) and b.finish_carrier(0) == 1 and "fused_on" not in b.kernel_source()
+            assert_y(b.spmv_device(x), y_ref, mag, npd, "carried finish, launches not fused")
+            b.set_fuse_launches(True)
+            b.compile().upload(gpu)
         assert_y(b.spmv_device(z), z_ref, z_mag, npd, "carried finish, second call with another x")
         assert_y(b.spmv_device(x, no_alloc=True), y_ref, mag, npd, "carried finish, static scratch")
         # one strip alone: its own kernels (the tile strip its finish kernel, the product-bin kernel nothing to carry)

@@ -56,6 +56,8 @@ def test_no_alloc_entry_point_matches_the_allocating_one(gpu, vdt, serial, carry
         print("case: no-alloc", name, b.rows, "serial" if serial else "concurrent", "carried" if carry else "own finish", flush=True)
         need = b.static_scratch_need()
         assert 0 < need <= STATIC_SCRATCH_BYTES
+        # both strips have workgroups of 1024 threads: with the carried finish their first kernels are one launch
+        assert b.launch_is_fused(0) == (serial and carry)
         y_alloc = b.spmv_device(x)
         y_static = b.spmv_device(x, no_alloc=True)
         _check(y_alloc, y_ref, mag, npd, name + ": as_builder_spmv_device against the oracle")
