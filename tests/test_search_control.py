@@ -87,7 +87,8 @@ def test_graph_report_shape():
     assert framed == "gflops:12.5\ntime:0.25\n" + H.graph_report(K.lib(), "as_", *H.GRAPH_CASES[0]) + "\nfinish search\n"
 
 
-def test_live_upstream_on_random_inputs():
+@EVERYWHERE
+def test_live_upstream_on_random_inputs(where):
     import ref_lib
     if not ref_lib.available():
         pytest.skip("oracle/_ref is not built here (upstream sources absent); the committed answers cover this")
