@@ -19,6 +19,12 @@ template <typename T> __device__ __forceinline__ T as_ldnt(const T *p) { return 
 // y is written once and not read again by the kernel: a streaming store keeps it from displacing x in L2
 template <typename T> __device__ __forceinline__ void as_stnt(T *p, T v) { __builtin_nontemporal_store(v, p); }
 
+// The workgroup's barrier, with every LDS operation of the wavefront complete before it.  The plain barrier alone was
+// compiled without the wait for outstanding LDS operations on one path into a barrier (a loop whose last iteration
+// jumps over the block that held the wait): sums that one wavefront had added to LDS were read by another before
+// they had landed.
+__device__ __forceinline__ void as_barrier() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); __syncthreads(); }
+
 __device__ __forceinline__ void as_atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
 __device__ __forceinline__ void as_atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 

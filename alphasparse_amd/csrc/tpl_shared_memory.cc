@@ -176,7 +176,7 @@ std::string kernel_source(const Template &t) {
   s += "        #pragma unroll 4\n        for (unsigned int k = 0; k < tlb_size; k++, nz += tlb_num)\n";
   s += "          acc += as_ldnt(val_arr + nz) * device_x_arr[" + fc + " + (unsigned int)as_ldnt(col_index_arr + nz)];\n";
   s += "        thread_tmp_result[first_tlb - block_first_tlb + u] = acc;\n      }\n    }\n";
-  s += "    __syncthreads();\n";
+  s += "    as_barrier();\n";
   s += "    for (unsigned int row = first_row + threadIdx.x / " + Rs + "u; row < next_first_row; row += " + B + "u / " + Rs + "u)\n    {\n";
   s += "      unsigned int next_row = row + 1u, res_begin, res_end;\n";
   s += "      " + code_of_meta_read(t, "row_offset_in_thread_tmp_result", "res_begin", "row");
@@ -193,7 +193,7 @@ std::string kernel_source(const Template &t) {
   s += t.is_atom_add ? "        as_atomic_add(device_y_arr + global_row_index, sum);\n"
                      : "        as_stnt(device_y_arr + global_row_index, sum);\n";
   s += "      }\n    }\n";
-  s += "    __syncthreads();\n  }\n}\n";
+  s += "    as_barrier();\n  }\n}\n";
   return s;
 }
 

@@ -103,7 +103,7 @@ std::string kernel_source(const Template &t) {
   s += "    acc = as_wave_sum(acc);\n";
   if (waves > 1) {
     s += "    if ((threadIdx.x & 63u) == 63u) wave_sum[threadIdx.x >> 6] = acc;\n";
-    s += "    __syncthreads();\n";
+    s += "    as_barrier();\n";
     s += "    if (threadIdx.x == 0)\n    {\n      acc = 0;\n";
     s += "      #pragma unroll\n      for (int w = 0; w < " + std::to_string(waves) + "; w++) acc += wave_sum[w];\n";
   } else {
@@ -116,7 +116,7 @@ std::string kernel_source(const Template &t) {
   s += t.is_atom_add ? "      as_atomic_add(device_y_arr + global_row_index, acc);\n"
                      : "      as_stnt(device_y_arr + global_row_index, acc);\n";
   s += "    }\n";
-  if (waves > 1) s += "    __syncthreads();\n";
+  if (waves > 1) s += "    as_barrier();\n";
   s += "  }\n}\n";
   return s;
 }

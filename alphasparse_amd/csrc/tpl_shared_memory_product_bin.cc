@@ -370,7 +370,7 @@ std::string kernel_source(const Template &t) {
     // trips of the shorter list would all land on the first XCDs.
     const std::string G0 = std::to_string(fused->tblock_num) + "u";
     s += "  if (fused_on && blockIdx.x < " + G0 + ")\n  {\n    " + kernel_trips_function_name(*fused) + "(" + kernel_arguments(*fused, "fused_") + ", blockIdx.x, " + G0 + ");\n";
-    s += "    __syncthreads();\n  }\n";   // the LDS is this kernel's from here on
+    s += "    as_barrier();\n  }\n";   // the LDS is this kernel's from here on
     s += "  const unsigned int as_block = blockIdx.x, as_grid = min(gridDim.x, " + std::to_string(t.tblock_num) + "u);\n";
     s += "  if (as_block >= as_grid) return;\n";
   } else {
@@ -396,7 +396,7 @@ std::string kernel_source(const Template &t) {
   s += "    const unsigned int bin0 = bins_before ? bins_before - 1u : 0u;\n";
   s += "    const unsigned int col0 = slice * " + Ss + ";\n";
   s += "    const unsigned int slice_len = min(" + Ss + ", " + std::to_string(x_len) + "u - col0);\n";
-  s += "    __syncthreads();\n";  // readers of the previous slice are done
+  s += "    as_barrier();\n";  // readers of the previous slice are done
   if (wide_copy) {
     // 16 bytes per lane and load (the 64 lanes of a load read one contiguous kilobyte); four loads of a lane
     // are requested before the first is stored
@@ -412,7 +412,7 @@ std::string kernel_source(const Template &t) {
     s += "    for (unsigned int i = threadIdx.x; i < slice_len; i += " + B + ") x_slice[i] = x_sub[col0 + i];\n";
   }
   s += "    for (unsigned int i = threadIdx.x; i < bins_end - bin0; i += " + B + ") shift_of_bin[i] = bin_shift[bin0 + i];\n";
-  s += "    __syncthreads();\n";
+  s += "    as_barrier();\n";
   // Consecutive lanes take consecutive elements: the products of a bin then go to consecutive places with one
   // store instruction (whole lines), instead of every fourth place with each of four.  A lane finds the bin of its
   // element by counting the flags of the elements before it: those of the unit's earlier loads (a scalar), those
@@ -486,7 +486,7 @@ std::string kernel_source(const Template &t) {
     s += "    " + code_of_meta_read(t, "band_first_row", "row_begin", "grp");
     s += "    " + code_of_meta_read(t, "band_first_row", "row_end", "next_grp");
   }
-  s += "    __syncthreads();\n";  // the previous band's sums have been read
+  s += "    as_barrier();\n";  // the previous band's sums have been read
   if (!table_in_register)
     s += "    for (unsigned int i = threadIdx.x; i <= width; i += " + FB + "u) first_slot[i] = band_slot_count[count_begin + i];\n";
   s += "    const unsigned int nz_end = unit_end * 256u;\n";
@@ -504,7 +504,7 @@ std::string kernel_source(const Template &t) {
   s += "        if (nz0 + k * stride >= nz_end) continue;\n";
   s += "        #pragma unroll\n        for (int j = 0; j < 4; j++) slots[(unsigned int)q[k][j]] = p[k][j];\n";
   s += "      }\n    }\n";
-  s += "    __syncthreads();\n";
+  s += "    as_barrier();\n";
   // Row sums: lane r0 + lane of a wavefront takes the row of that rank; rows are ranked by falling length, so the
   // wavefront is done where its first row is (a test on scalars).  Rows without elements have the last ranks.
   // Four elements of a row are requested from LDS before the first is added.
@@ -529,7 +529,7 @@ std::string kernel_source(const Template &t) {
     // slot r is the row's own first element: nobody else reads it
     s += "      if (r < live) slots[r] = sum;\n";
     s += "    }\n";
-    s += "    __syncthreads();\n";
+    s += "    as_barrier();\n";
     s += "    #pragma unroll\n    for (int k = 0; k < " + As + "; k++)\n    {\n";
     s += "      const unsigned int i = threadIdx.x + k * " + FB + "u;\n";
     s += "      if (i < height && rank[k] != " + std::to_string(kNoRank) + "u)\n";

@@ -626,7 +626,7 @@ std::string kernel_source(const Template &t) {
   s += "    " + code_of_meta_read(t, "group_first_run", "run_begin", "grp");
   s += "    " + code_of_meta_read(t, "group_first_run", "run_end", "next_grp");
   s += "    run_begin = __builtin_amdgcn_readfirstlane(run_begin); run_end = __builtin_amdgcn_readfirstlane(run_end);\n";
-  s += "    __syncthreads();\n";  // the previous trip's write-back is done with the cells
+  s += "    as_barrier();\n";  // the previous trip's write-back is done with the cells
   s += "    for (unsigned int i = threadIdx.x; i < " + Rs + "; i += " + B + ") piece_sum[i] = 0;\n";
   if (t.own_rows) s += "    unsigned int cur_slice = 0xffffffffu, cur_group = 0xffffffffu;\n";
   else s += "    unsigned int cur_slice = 0xffffffffu, done_begin = 0u, done_end = 0u;\n";
@@ -644,7 +644,7 @@ std::string kernel_source(const Template &t) {
     s += "        " + code_of_meta_read(t, "run_piece_begin", "piece_end", "next_run");
   }
   s += "      }\n";
-  s += "      __syncthreads();\n";  // every wavefront is done with the previous run
+  s += "      as_barrier();\n";  // every wavefront is done with the previous run
   // Between two runs a workgroup writes the finished run back (a table read and one atomic per piece) and, when the
   // slice changes, copies the new slice of x into LDS.  Written as plain loops, both are chains of memory round
   // trips: the compiler waits for an atomic to complete before it lets anything overwrite the atomic's data
@@ -716,7 +716,7 @@ std::string kernel_source(const Template &t) {
     s += "        }\n";
   }
   s += "        cur_slice = slice;\n      }\n";
-  s += "      __syncthreads();\n";
+  s += "      as_barrier();\n";
   // Runs are padded to whole wavefront steps: a step is inside the run for all lanes or for none, and the steps
   // outside are neither loaded nor used.  All loads of a full batch are requested before the first is used.
   auto load_step = [&](const std::string &ind) {

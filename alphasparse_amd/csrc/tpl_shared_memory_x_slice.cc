@@ -168,7 +168,7 @@ std::string kernel_source(const Template &t) {
   s += "    " + code_of_meta_read(t, "group_first_unit", "next_first_unit", "next_grp");
   s += "    const unsigned int col0 = slice * " + Ss + ";\n";
   s += "    const unsigned int slice_len = min(" + Ss + ", " + std::to_string(x_len) + "u - col0);\n";
-  s += "    __syncthreads();\n";   // readers of the previous slice are done
+  s += "    as_barrier();\n";   // readers of the previous slice are done
   // full slices are copied with a fixed trip count so that all loads of a lane are in flight together
   const uint64_t copy_trips = (S + 4 * t.thread_num_in_block - 1) / (4 * t.thread_num_in_block);
   s += "    if (slice_len == " + Ss + ")\n    {\n";
@@ -184,7 +184,7 @@ std::string kernel_source(const Template &t) {
   s += "        *(val4_t *)(x_slice + i) = *(const val4_t *)(x_sub + col0 + i);\n";
   s += "      if (threadIdx.x < (slice_len & 3u)) x_slice[(slice_len & ~3u) + threadIdx.x] = x_sub[col0 + (slice_len & ~3u) + threadIdx.x];\n";
   s += "    }\n";
-  s += "    __syncthreads();\n";
+  s += "    as_barrier();\n";
   // K steps of 4 units per trip: all loads of the K steps are issued before the first use
   const std::string Ks = std::to_string(kBatch);
   s += "    for (unsigned int ub = first_unit + wave_in_block * 4u; ub < next_first_unit; ub += wave_num * 4u * " + Ks + "u)\n    {\n";

@@ -252,7 +252,7 @@ std::string kernel_source(const Template &t) {
   s += "      " + code_of_meta_read(t, "global_warp_block_first_nz", "nz_end", "next_wlb");
   s += code_of_wlb_dot(t, "      ");
   s += "      if (lane == 63u) warp_tmp_result[wlb - first_wlb] = acc;\n    }\n";
-  s += "    __syncthreads();\n";
+  s += "    as_barrier();\n";
   // rows of the BLB: groups of R lanes add the WLB sums of one row
   s += "    for (unsigned int row = first_row + threadIdx.x / " + Rs + "u; row < next_first_row; row += " + B + "u / " + Rs + "u)\n    {\n";
   s += "      unsigned int next_row = row + 1u, res_begin, res_end;\n";
@@ -271,7 +271,7 @@ std::string kernel_source(const Template &t) {
   s += t.is_atom_add ? "        as_atomic_add(device_y_arr + global_row_index, sum);\n"
                      : "        as_stnt(device_y_arr + global_row_index, sum);\n";
   s += "      }\n    }\n";
-  s += "    __syncthreads();\n  }\n}\n";
+  s += "    as_barrier();\n  }\n}\n";
   return s;
 }
 

@@ -945,3 +945,28 @@ def test_remove_empty_rows_and_sort_through_the_map():
     before = m2.info()["rows"]
     m2.remove_empty_rows()
     assert m2.info()["rows"] == before and "sorted_row_index" not in m2.dump()
+
+
+def test_every_barrier_of_the_generated_kernels_waits_for_the_wavefronts_lds_operations():
+    """Every workgroup barrier in the generated kernels is as_barrier(): the wait for the wavefront's outstanding LDS
+    operations is written out in front of it.  (The compiler left that wait out on one path into a barrier of the
+    fused tile + product-bin kernel -- the last iteration of the loop over a trip's runs -- and rows of the tile
+    strip then lost the sums of a trip's last run now and then.)"""
+    import os
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
+    import __graft_entry__ as G
+    from alphasparse_amd import skeletons as SK
+    mats = {"power_law": S.power_law(512, max_len=200, mean_len=12.0, seed=11), "uniform": S.uniform_rows(512, 40, seed=12)}
+    with_lds = 0
+    for mat, skel, kw in G.kernel_build_cases():
+        rows, cols, r, c, v, _ = mats[mat]
+        m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.FLOAT, wave=64)
+        m.execute_strategy(K.COMPRESS_NONE)
+        for template in SK.apply_skeleton(m, 0, skel, **kw):
+            b = A.Builder(m)
+            b.set_template(0, template)
+            src = b.kernel_source()
+            assert src.count("__syncthreads()") == 1 and "s_waitcnt lgkmcnt(0)" in src.split("__syncthreads()")[0].splitlines()[-1], K.TEMPLATE_NAMES[template]
+            with_lds += "as_barrier();" in src
+    assert with_lds >= 6

@@ -105,3 +105,59 @@ def test_random_two_strip_graphs_with_the_finish_carried(gpu):
         b.time(3)
         _check(b, x, y_ref, mag, npd, what + ", after a timing loop")
         b.close()
+
+
+def test_random_two_strip_graphs_in_one_launch(gpu):
+    """The same shape of graph with workgroups of one size in both strips, so that the tile trips and the first pass of
+    the product-bin template are one launch and the second pass carries the tile strip's finish.  Rows of two classes
+    of length in random proportion: where the short rows are the minority the product-bin template keeps the rows of y
+    by rank (sparse form) instead of a rank for every row of y; rows without a short neighbour, bands of y that the
+    strip does not touch, more tile trips than first-pass trips and the other way round all come up.  Fused and not
+    fused against the oracle, y = NaN before every call, again after a timing loop."""
+    import cases
+    fused = sparse = 0
+    for case in range(18):
+        rng = np.random.default_rng(700 + case)
+        rows = int(rng.integers(3000, 90000))
+        share_short = float(rng.choice([0.15, 0.4, 0.7, 0.95]))
+        short = rng.integers(1, int(rng.choice([4, 9, 15])), rows)
+        long_ = rng.integers(16, int(rng.choice([64, 400, 2500])), rows)
+        lens = np.where(rng.random(rows) < share_short, short, long_)
+        if lens.sum() > 6_000_000:      # keep the case small: shorter long rows, still 16 or more elements
+            lens = np.where(lens >= 16, np.maximum(16, lens * 6_000_000 // lens.sum()), lens)
+        cols = int(rng.choice([rows, 2 * rows, 70000]))
+        vdt = K.DOUBLE if rng.integers(2) else K.FLOAT
+        s1, g1 = int(rng.choice([512, 1024, 4096])), int(rng.choice([128, 512, 2048]))
+        s2, g2 = int(rng.choice([512, 1024, 4096])), int(rng.choice([256, 1024, 4096]))
+        threads = int(rng.choice([256, 512, 1024]))
+        what = "case %d: %d rows x %d columns, %.0f %% short rows, tile %d x %d, product-bin %d x %d, %d threads, %s" % (
+            case, rows, cols, 100 * share_short, g1, s1, g2, s2, threads, "fp64" if vdt == K.DOUBLE else "fp32")
+        print(what, flush=True)
+        rows, cols, r, c, v, x = cases._steps(lens, max(cols, int(lens.max())), 700 + case)
+        npd = np.float64 if vdt == K.DOUBLE else np.float32
+        v, x = v.astype(npd), x.astype(npd)
+        m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
+        m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+        m.execute_strategy(K.DENSE_ROW_DIV_ACC_TO_EXPONENTIAL_INCREASE_ROW_NNZ, -1, (16, 16, 2, 0))
+        m.execute_strategy(K.COMPRESS_NONE)
+        assert m.info()["n_sub"] == 2
+        b = A.Builder(m)
+        b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=s1, group=g1, b=2048)[0])
+        b.set_template(1, SK.apply_skeleton(m, 1, "T2", slice=s2, group=g2, b=2048)[0])
+        b.set_launch(0, thread_num_in_block=threads)
+        b.set_launch(1, thread_num_in_block=threads)
+        b.set_serial_launch(True)
+        b.compile().upload(gpu)
+        assert b.launch_is_fused(0) and b.finish_carrier(0) == 1
+        fused += 1
+        sparse += b.describe(1)["dense_y"] == 0
+        y_ref, mag = O.spmv_csr(O.coo_to_csr(rows, r), c.astype(np.uint32), v, x)
+        _check(b, x, y_ref, mag, npd, what)
+        b.time(3)
+        _check(b, x, y_ref, mag, npd, what + ", after a timing loop")
+        b.set_fuse_launches(False)
+        b.compile().upload(gpu)
+        assert not b.launch_is_fused(0) and b.finish_carrier(0) == 1
+        _check(b, x, y_ref, mag, npd, what + ", launches not fused")
+        b.close()
+    assert fused == 18 and sparse >= 3, (fused, sparse)
