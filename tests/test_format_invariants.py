@@ -970,3 +970,38 @@ def test_every_barrier_of_the_generated_kernels_waits_for_the_wavefronts_lds_ope
             assert src.count("__syncthreads()") == 1 and "s_waitcnt lgkmcnt(0)" in src.split("__syncthreads()")[0].splitlines()[-1], K.TEMPLATE_NAMES[template]
             with_lds += "as_barrier();" in src
     assert with_lds >= 6
+
+
+def test_tile_trips_fit_one_round_of_workgroups():
+    """The tile template cuts its element stream into trips between BLBs; however the cuts fall, there are never more
+    trips than workgroups the device holds at a time with the template's LDS need (one more would wait for a second
+    round and the kernel would take nearly twice as long).  Cases 16, 99, 113 and 127 came out one to six trips above
+    that before the share of a trip was raised until the trips fit."""
+    from alphasparse_amd import skeletons as SK
+    at_the_limit = 0
+    try:
+        for case in (16, 99, 113, 127, 0, 1, 3, 4, 5, 6, 7, 8):
+            rng = np.random.default_rng(9000 + case)
+            cus = int(rng.choice([8, 16, 24, 64]))
+            A.device_facts(cu_num=cus)
+            rows = int(rng.integers(2000, 30000))
+            mult = int(rng.integers(1, 40))
+            lens = np.minimum(rng.zipf(1.7, rows) * mult, 3000)
+            rows, cols, r, c, v, x = cases._steps(lens, max(rows, int(lens.max())), 9000 + case)
+            m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), K.FLOAT, wave=64)
+            if rng.integers(2):
+                m.execute_strategy(K.DENSE_ROW_COARSE_SORT_FIXED, -1, (1,))
+            m.execute_strategy(K.COMPRESS_NONE)
+            slice_width, group = int(rng.choice([1024, 4096, 16384, 32768])), int(rng.choice([512, 2048, 4096, 6144]))
+            blb = int(rng.choice([64, 256, 1024, 8192]))
+            b = A.Builder(m)
+            b.set_template(0, SK.apply_skeleton(m, 0, "T1", slice=slice_width, group=group, b=blb)[0])
+            per_cu = max(1, 163840 // ((slice_width + group) * 4))
+            trips = b.describe(0)["group_num"]
+            assert 1 <= trips <= cus * per_cu, (case, trips, cus, per_cu)
+            assert b.get_launch(0)["tblock_num"] == trips
+            at_the_limit += trips > 0.9 * cus * per_cu
+            b.close()
+    finally:
+        A.device_facts(reset=True)
+    assert at_the_limit >= 6      # the cases do reach the limit
