@@ -9,8 +9,12 @@
 //
 //   spmv_<sub>         slice by slice: a workgroup copies its slice of x into LDS, multiplies every
 //                      element of its trip by its x value (LDS read) and writes the product to the
-//                      place the element has in band order (a stored 32-bit position; the elements of
-//                      a (slice, band) bin stay together, so the writes come in runs);
+//                      place the element has in band order: the element's own number plus the shift of
+//                      its bin (the elements of one band in one slice; they stay together, so the
+//                      writes come in runs).  The top bit of the 16-bit column marks the first element
+//                      of a bin; a lane finds its bin by counting the marks in front of its element
+//                      (a table gives the count at the start of every 256 elements, a ballot and a bit
+//                      count the rest), the shifts of the trip's bins wait in LDS beside the slice;
 //   spmv_<sub>_finish  band by band: one workgroup owns the band, streams its products (contiguous)
 //                      and drops each into its own LDS slot -- the j-th element of the row of rank r
 //                      goes to slot first[j] + r, where first[j] counts the slots of the elements
@@ -25,9 +29,9 @@
 //                      Where the strip holds few of the rows of y its bands span (less than half), the
 //                      lane that summed a row stores it through a 16-bit place inside the band instead.
 //
-// Per element: value + 16-bit column inside the slice + 32-bit position (first pass), 16-bit LDS slot
-// (second pass), and the product written once and read once; per row of y 16 bits.  No access to HBM
-// is a gather.
+// Per element: value + 16-bit column inside the slice (first pass), 16-bit LDS slot (second pass), and the
+// product written once and read once; per bin a 32-bit shift, per row of y 16 bits.  No access to HBM is a
+// gather.
 #include "device_facts.hpp"
 #include "templates.hpp"
 
