@@ -642,9 +642,11 @@ def test_full_size_tile_and_product_bin_graphs(gpu, make, capsys):
 def test_finish_of_a_tile_strip_carried_by_the_next_strips_kernel(gpu, vdt):
     """Coarse sort, a tile strip (row sums through a scratch vector and a finish kernel) in front of a product-bin
     strip, kernels one after the other: the finish kernel is not launched, the first workgroups of the product-bin
-    template's first kernel move the rows to y.  y against the oracle with the hand-over on and off, on y = NaN, call
-    after call (the scratch vector is left cleared), after measurements of one strip alone (which use the strip's
-    own kernels), and on concurrent streams (no hand-over)."""
+    template's first kernel move the rows to y -- or, where both strips have workgroups of the same size, the two
+    strips' first kernels are one launch and the product-bin template's second kernel moves the rows.  y against the
+    oracle with the hand-over on and off, fused and not, on y = NaN, call after call (the scratch vector is left
+    cleared), after measurements of one strip alone (which use the strip's own kernels), and on concurrent streams
+    (no hand-over)."""
     rows, cols, r, c, v, x = S.power_law(30000, max_len=4000, mean_len=12.0, seed=11)
     npd = NP[vdt]
     v, x = v.astype(npd), x.astype(npd)
