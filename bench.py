@@ -20,7 +20,10 @@ whole SpMV; with more than one row strip `roofline.dominant_kernel` holds the st
 timed alone, and "kernels" lists every strip kernel.  Two byte counts are given side by side: `algorithmic_bytes` /
 `frac` count what the chosen format moves, the intermediate arrays its kernels write and read back included
 (products, row sums: `scratch_bytes`, counted twice); `algorithmic_bytes_arrays_x_y` / `frac_arrays_x_y` count the
-format arrays, x once and y once only (twice where y is cleared first).
+format arrays, x once and y once only (twice where y is cleared first).  `per_call_us` is one SpMV four ways: between
+events on the stream (`kernels`, what `value` is made of), as a blocking product call, as an enqueue-only product
+call, and as a replay of the allocation-free enqueue-only call captured into a HIP graph (null where the kernels'
+scratch arrays do not fit the library's static array).
 
 Prints ONE JSON line (rank 0).  One GPU only: --gpus above 1 exits with a message."""
 import argparse
@@ -248,6 +251,34 @@ def measure(key, steps, warmup, tune_seconds, pin, cpu_seconds, copy_calibration
         b.spmv_device_async(dx, dy, None)
     b.sync()
     per_call_async_us = (time.perf_counter() - t0) / calls * 1e6
+    # ... and the allocation-free enqueue-only call recorded once by a stream capture and replayed as a HIP graph
+    # (null where the kernels' scratch arrays do not fit the library's static array)
+    per_call_graph_us = None
+    try:
+        if 0 <= b.static_scratch_need() <= (64 << 20):
+            stream = A.Stream()
+            b.spmv_device_async(dx, dy, stream, no_alloc=True)
+            stream.sync()
+            stream.capture_begin()
+            b.spmv_device_async(dx, dy, stream, no_alloc=True)
+            graph = stream.capture_end()
+            for _ in range(20):
+                stream.graph_launch(graph)
+            stream.sync()
+            t0 = time.perf_counter()
+            for _ in range(calls):
+                stream.graph_launch(graph)
+            stream.sync()
+            per_call_graph_us = (time.perf_counter() - t0) / calls * 1e6
+            y_graph = dy.get()
+            rel_g, ratio_g, tol_g = O.check_y(y_graph, *O.spmv_csr(O.coo_to_csr(rows, r), c.astype(np.uint32), v, x), v.dtype.type)
+            if not (rel_g <= tol_g and ratio_g <= 1.0):
+                raise RuntimeError("%s: the replayed graph's y differs (rel L2 %.3e)" % (key, rel_g))
+            stream.graph_destroy(graph)
+            stream.destroy()
+    except A.AlphaSparseError as e:
+        print("[bench] %s: graph replay not timed: %s" % (key, str(e)[:200]), file=sys.stderr)
+        per_call_graph_us = None
     dx.free()
     dy.free()
     scratch = b.scratch_bytes()
@@ -300,7 +331,8 @@ def measure(key, steps, warmup, tune_seconds, pin, cpu_seconds, copy_calibration
                        "frac_arrays_x_y": round(bytes_arrays_x_y / per_launch_s / 1e9 / HBM_PEAK_GBS, 4),
                        "kernel_gflops": round(2.0 * nnz / per_launch_s / 1e9, 2)},
         "per_call_us": {"kernels": round(per_launch_s * 1e6, 3), "blocking_call": round(per_call_sync_us, 3),
-                        "enqueue_only_call": round(per_call_async_us, 3), "calls": calls},
+                        "enqueue_only_call": round(per_call_async_us, 3),
+                        "graph_replay": None if per_call_graph_us is None else round(per_call_graph_us, 3), "calls": calls},
         "kernels": kernels,
         "tuning": {"mode": "pinned" if pin else "search", "seconds": round(tune_s, 2),
                    "seconds_to_best": round(res.seconds_to_best, 2),
