@@ -128,9 +128,12 @@ def test_no_alloc_async_call_replayed_as_a_hip_graph(gpu, vdt):
     clears with fill kernels, not memset nodes) and replayed three times with a different x each time, the program's
     own eager work and waits in between: every replay must give A x for the x of that replay.  Two graphs: the
     two-strip graph (scratch of both strips in the static array, the tile strip's piece cleared by the fill kernel,
-    finish carried) and a graph that starts with a clear of y."""
+    finish carried), the same with the strips on concurrent streams (the capture records the fork and the join) and
+    a graph that starts with a clear of y."""
     npd = NP[vdt]
-    cases = [_two_strip_builder(gpu, 20000, 3000, 31, vdt)]
+    cases = [_two_strip_builder(gpu, 20000, 3000, 31, vdt),
+             # the strips' kernels on streams of their own, which fork from and join the capturing stream by events
+             _two_strip_builder(gpu, 12000, 2000, 33, vdt, serial=False)]
     rows, cols, r, c, v, x = S.power_law(8000, max_len=900, mean_len=20.0, seed=5)
     m = A.Matrix.from_coo(rows, cols, r, c, v.astype(np.float64), vdt, wave=64)
     m.execute_strategy(K.COMPRESS_NONE)
