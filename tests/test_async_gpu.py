@@ -84,3 +84,30 @@ def test_a_hundred_enqueued_calls_then_one_wait(gpu, vdt, no_alloc):
                 d.free()
         b.close()
     stream.destroy()
+
+
+def test_enqueue_only_call_on_the_default_stream(gpu):
+    """A null stream argument is HIP's default stream (not the builder's own): calls through the C-ABI with NULL, a
+    device-wide wait, y against the oracle -- for the two-strip graph one after the other and on concurrent streams
+    (which then fork from and join the default stream)."""
+    import ctypes as C
+    L = K.lib()
+    for serial in (True, False):
+        name, b, rows, cols, r, c, v = graphs(gpu, K.FLOAT)[1]
+        b.set_serial_launch(serial)
+        b.compile().upload(gpu)
+        rng = np.random.default_rng(3)
+        row_ptr, col32 = O.coo_to_csr(rows, r), np.asarray(c).astype(np.uint32)
+        dx, dy = A.DeviceArray(np.zeros(cols, np.float32)), A.DeviceArray(np.full(rows, np.nan, np.float32))
+        for call in range(5):
+            x = rng.uniform(-1, 1, cols).astype(np.float32)
+            dx.set(x)
+            for no_alloc in (False, True):
+                f = L.as_builder_spmv_device_no_alloc_async if no_alloc else L.as_builder_spmv_device_async
+                K.check(f(b._h, dx.ptr, dy.ptr, C.c_void_p(None)), L)
+                assert L.as_hip_device_sync() == 0
+                y_ref, mag = O.spmv_csr(row_ptr, col32, v, x)
+                _check(dy.get(), y_ref, mag, np.float32, "default stream, call %d, %s, %s" % (call, "serial" if serial else "concurrent", "no_alloc" if no_alloc else "alloc"))
+        dx.free()
+        dy.free()
+        b.close()
